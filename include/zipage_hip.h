@@ -1,0 +1,170 @@
+/* C ABI of libzipage_hip.so: hand-written gfx950 (MI355X) kernels for the KV-cache
+ * compression path of compressed PagedAttention.
+ *
+ * The reference (microsoft/Zipage) has no FFI on this path: its boundary is the set of
+ * Python functions under zipage/kernel/.  Each entry point below replaces the device
+ * work of one of them and is what a Python (ctypes) or C++ host binds; the citation on
+ * each declaration names the reference interface it stands in for.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller; nothing is retained;
+ *   - dims are int32, strides are int64 and counted in ELEMENTS; the innermost
+ *     (head_dim / slot) axis of every tensor has stride 1;
+ *   - `dtype` tags the element type of caches and scores (zp_dtype);
+ *   - `stream` is a hipStream_t passed as void*; calls only enqueue work on it, never
+ *     synchronise the device and never allocate;
+ *   - functions return ZP_OK or an error code; zp_last_error() gives the thread-local
+ *     message of the last failure on the calling thread;
+ *   - block tables are contiguous int32 (B, NB): id >= 0 full page, -1 padding,
+ *     x < -1 the sequence's last page with id = -x-2
+ *     (zipage/engine/model_runner.py:437-463);
+ *   - a page id outside [0, num_pages) is treated as padding instead of being
+ *     dereferenced.
+ */
+#ifndef ZIPAGE_HIP_H
+#define ZIPAGE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { ZP_BF16 = 0, ZP_F16 = 1, ZP_F32 = 2 } zp_dtype;
+
+enum { ZP_OK = 0, ZP_EINVAL = 1, ZP_EHIP = 2, ZP_EUNSUPPORTED = 3 };
+
+enum { ZP_REDUCE_MEAN = 0, ZP_REDUCE_MAX = 1 };    /* attention_score `reduced` */
+enum { ZP_ACTIVATE_MAX = 0, ZP_ACTIVATE_SUM = 1 }; /* global_score `activate_method` */
+enum { ZP_POOL_MAX = 0, ZP_POOL_AVG = 1 };
+
+/* ABI version of this header; bumped on any signature change. */
+int zp_abi_version(void);
+/* Message of the last error raised on the calling thread ("" if none). */
+const char* zp_last_error(void);
+
+/* store_query_cache(query, query_cache, slot_mapping)
+ * zipage/kernel/store_query_cache.py:35-68 (kernel :7-32).
+ * For each of the n int32 triples (pos, seq_id, slot):
+ *   query_cache[seq_id, slot, :] = query[pos, :]   (row_elems = Hq*D elements). */
+int zp_store_query(const void* query, void* query_cache, const int32_t* slot_mapping,
+                   int32_t n, int32_t row_elems, int32_t num_tokens, int32_t max_seqs,
+                   int32_t window, int64_t q_stride_tok, int64_t c_stride_seq,
+                   int64_t c_stride_slot, int64_t sm_stride_row, int64_t sm_stride_col,
+                   int32_t dtype, void* stream);
+
+/* attention_score(k_cache, query_cache, seq_idx, block_table, softmax_scale, reduced,
+ *                 return_logits)
+ * zipage/kernel/attention_score.py:133-250 (kernel :8-130).
+ * k_cache (L, num_pages, BS, Hkv, D), query_cache (L, max_seqs, W, Hq, D), both
+ * contiguous in their last two axes; scores_out (L, B, Hkv, NB, BS) contiguous, in the
+ * cache dtype; logits_out NULL or (L, B, Hq, W, NB, BS) contiguous.
+ * workspace: zp_attention_score_workspace() bytes of device scratch. */
+int zp_attention_score(const void* k_cache, const void* query_cache, const int32_t* seq_idx,
+                       const int32_t* block_table, void* scores_out, void* logits_out,
+                       int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
+                       int32_t Hq, int32_t D, int32_t W, int32_t num_pages,
+                       int32_t max_seqs, int64_t k_stride_layer, int64_t k_stride_page,
+                       int64_t q_stride_layer, int64_t q_stride_seq, float softmax_scale,
+                       int32_t reduced, int32_t dtype, void* workspace,
+                       int64_t workspace_bytes, void* stream);
+int64_t zp_attention_score_workspace(int32_t L, int32_t B, int32_t NB, int32_t BS,
+                                     int32_t Hkv, int32_t Hq, int32_t W);
+
+/* global_score(reduced_scores, score_cache, block_table, compressed, decay_factor,
+ *              activate_method)
+ * zipage/kernel/global_score.py:77-120 (kernel :8-74).
+ * scores (L, B, Hkv, NB, BS) contiguous, updated in place; score_cache
+ * (L, num_pages, BS, Hkv) with the given layer/page strides, slot stride Hkv, head
+ * stride 1; compressed: B bytes (bool). */
+int zp_global_score(void* scores, void* score_cache, const int32_t* block_table,
+                    const uint8_t* compressed, int32_t L, int32_t B, int32_t NB,
+                    int32_t BS, int32_t Hkv, int32_t num_pages, int64_t c_stride_layer,
+                    int64_t c_stride_page, float decay_factor, int32_t activate_method,
+                    int32_t dtype, void* stream);
+
+/* Sequence-axis pooling done inline by the runner:
+ * zipage/engine/model_runner.py:499-530  (F.max_pool1d, stride 1, pad kernel//2, then
+ * torch.where(compressed, raw, pooled) unless continues_pooling).
+ * in/out (L, B, Hkv, T) contiguous, distinct buffers.  ZP_POOL_AVG is an extension
+ * with no counterpart in the reference. */
+int zp_pool_scores(const void* scores_in, void* scores_out, const uint8_t* compressed,
+                   int32_t L, int32_t B, int32_t Hkv, int32_t T, int32_t kernel_size,
+                   int32_t continues_pooling, int32_t mode, int32_t dtype, void* stream);
+
+/* key_norm(key_cache, block_table, norm_epsilon)
+ * zipage/kernel/key_norm.py:72-113 (kernel :8-69).  norm_out (L,B,Hkv,NB,BS). */
+int zp_key_norm(const void* k_cache, const int32_t* block_table, void* norm_out, int32_t L,
+                int32_t B, int32_t NB, int32_t BS, int32_t Hkv, int32_t D,
+                int32_t num_pages, int64_t k_stride_layer, int64_t k_stride_page,
+                float norm_epsilon, int32_t dtype, void* stream);
+
+/* lightning_redudancy_score / raw_redudancy_score(key_cache, block_table, threshold,
+ *                                                 temperature, return_logits)
+ * zipage/kernel/lightning_redudancy_score.py:172-261 (kernel :10-169)
+ * zipage/kernel/raw_redudancy_score.py:158-238 (kernel :10-155).
+ * red_out (L,B,Hkv,NB,BS) softmax-normalised redundancy; logits_out NULL or the same
+ * shape with the pre-softmax row sums (pad pages -inf). */
+int zp_redundancy_lightning(const void* k_cache, const int32_t* block_table, void* red_out,
+                            void* logits_out, int32_t L, int32_t B, int32_t NB, int32_t BS,
+                            int32_t Hkv, int32_t D, int32_t num_pages,
+                            int64_t k_stride_layer, int64_t k_stride_page, float threshold,
+                            double temperature, int32_t dtype, void* stream);
+int zp_redundancy_raw(const void* k_cache, const int32_t* block_table, void* red_out,
+                      void* logits_out, int32_t L, int32_t B, int32_t NB, int32_t BS,
+                      int32_t Hkv, int32_t D, int32_t num_pages, int64_t k_stride_layer,
+                      int64_t k_stride_page, float threshold, double temperature,
+                      int32_t dtype, void* workspace, int64_t workspace_bytes,
+                      void* stream);
+int64_t zp_redundancy_raw_workspace(int32_t L, int32_t B, int32_t NB, int32_t BS,
+                                    int32_t Hkv);
+
+/* Score post-processing done inline by the runner, fused into one pass over
+ * (L, B, Hkv, NB*BS), in place on `scores`:
+ *   zipage/engine/model_runner.py:482-487  scores /= max_T            (max_norm_scores)
+ *   zipage/engine/model_runner.py:551-559  red /= max_T (max_norm_red);
+ *                                          scores*lambda - red*(1-lambda)  (red != NULL)
+ *   zipage/engine/model_runner.py:565-578  first sink_len tokens -> +inf   (sink_len>0)
+ *   zipage/kernel/window_mask.py:47-72     last `window` slots of the last page -> +inf
+ *                                          (window > 0)
+ *   zipage/engine/model_runner.py:592-593  pad pages -> -inf               (mask_pad)
+ * Any subset can be selected; window_mask() alone is window>0 with everything else off.
+ */
+int zp_score_epilogue(void* scores, const void* redundancy, const int32_t* block_table,
+                      int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
+                      int32_t max_norm_scores, int32_t max_norm_red, double redudancy_lambda,
+                      int32_t sink_len, int32_t window, int32_t mask_pad, int32_t dtype,
+                      void* stream);
+
+/* topk_mask(scores, k)   zipage/kernel/utils.py:21-36.
+ * scores (rows, T) contiguous; flag_out (rows, T) bytes, exactly min(k,T) ones per row.
+ * Ties are broken towards the lowest index (torch.topk leaves them unspecified). */
+int zp_topk_mask(const void* scores, uint8_t* flag_out, int32_t rows, int32_t T, int32_t k,
+                 int32_t dtype, void* stream);
+
+/* compress_kv(key, value, flag, block_table, target_block_table)
+ * zipage/kernel/compress_kv.py:103-141 (kernel :8-100).
+ * key/value (L, num_pages, BS, Hkv, D) with the given element strides (head_dim stride
+ * 1); flag (L, B, Hkv, NB, BS) bytes contiguous; target (B, target_width) int32.
+ * Stable in-place compaction; a target page may alias a source page of the same
+ * sequence at the same or a lower logical index. */
+int zp_compress_kv(void* key, void* value, const uint8_t* flag, const int32_t* block_table,
+                   const int32_t* target_block_table, int32_t L, int32_t B, int32_t NB,
+                   int32_t BS, int32_t Hkv, int32_t D, int32_t num_pages,
+                   int32_t target_width, int64_t k_stride_layer, int64_t k_stride_page,
+                   int64_t k_stride_slot, int64_t k_stride_head, int64_t v_stride_layer,
+                   int64_t v_stride_page, int64_t v_stride_slot, int64_t v_stride_head,
+                   int32_t dtype, void* stream);
+
+/* compress_score(score_cache, flag, block_table, target_block_table)
+ * zipage/kernel/compress_score.py:66-99 (kernel :8-63). */
+int zp_compress_score(void* score_cache, const uint8_t* flag, const int32_t* block_table,
+                      const int32_t* target_block_table, int32_t L, int32_t B, int32_t NB,
+                      int32_t BS, int32_t Hkv, int32_t num_pages, int32_t target_width,
+                      int64_t c_stride_layer, int64_t c_stride_page, int64_t c_stride_slot,
+                      int64_t c_stride_head, int32_t dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ZIPAGE_HIP_H */

@@ -1,0 +1,314 @@
+"""GPU parity: every HIP entry point against the CPU oracle on the same seeded inputs.
+
+Bars: bit-exact for copies, masks and indices; for floating-point scores 1e-3 relative
+(plus a small absolute floor) with fp32 caches, and at most one unit in the last place of
+the cache dtype with bf16/fp16 caches (the reference rounds its intermediates to the cache
+dtype, so 1e-3 is below the output's own resolution there).
+"""
+import pytest
+import torch
+
+from oracle import zipage_oracle as O
+from tests import cases
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+
+
+def _ulp_close(got, want, dtype, ulps=1, frac_exact=0.0):
+    """got/want: tensors in `dtype`.  Every element within `ulps` units in the last place."""
+    g, w = got.float().cpu(), want.float().cpu()
+    assert torch.equal(torch.isinf(g), torch.isinf(w))
+    fin = torch.isfinite(w)
+    g, w = g[fin], w[fin]
+    eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -24}[dtype]
+    tol = ulps * 2 * eps * torch.maximum(w.abs(), g.abs()) + 1e-30
+    bad = (g - w).abs() > tol
+    assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} beyond {ulps} ulp; max diff {(g - w).abs().max()}"
+    if frac_exact:
+        same = (g == w).float().mean().item()
+        assert same >= frac_exact, f"only {same:.4f} bit-identical"
+
+
+def _rel_close(got, want, rel=1e-3, abs_floor=1e-7):
+    g, w = got.float().cpu(), want.float().cpu()
+    assert torch.equal(torch.isinf(g), torch.isinf(w))
+    fin = torch.isfinite(w)
+    err = (g[fin] - w[fin]).abs()
+    tol = rel * w[fin].abs() + abs_floor
+    assert (err <= tol).all(), f"max rel err {(err / (w[fin].abs() + abs_floor)).max()}"
+
+
+def _setup(seed, dtype, L=2, B=3, Hkv=2, Hq=8, D=128, W=32, BS=256, nb_choices=(3, 4), budget=2,
+           num_pages=24, score_cache=False):
+    tables, enc, target = cases.random_tables(seed, B, num_pages, list(nb_choices), budget)
+    k, v, q, sc = cases.make_caches(seed, L, num_pages, BS, Hkv, Hq, D, W, B + 2, dtype,
+                                    touched=cases.touched_pages(enc), with_score_cache=score_cache)
+    seq_idx = torch.tensor([(b * 2 + 1) % (B + 2) for b in range(B)], dtype=torch.int32)
+    return dict(k=k, v=v, q=q, sc=sc, enc=enc, target=target, seq_idx=seq_idx, tables=tables)
+
+
+# ------------------------------------------------------------------ copies / masks
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_store_query_cache(dev, dtype):
+    from zipage_amd.kernel import store_query_cache
+    g = torch.Generator().manual_seed(3)
+    Ntok, Hq, D, W, S = 37, 8, 128, 16, 5
+    q = torch.randn((Ntok, Hq, D), generator=g).to(dtype)
+    qc = torch.randn((S, W, Hq, D), generator=g).to(dtype)
+    sm = torch.tensor([[0, 1, 3], [36, 4, 15], [7, 0, 0], [8, 0, 1], [20, 2, 9]], dtype=torch.int32)
+    want = qc.clone()
+    O.store_query_cache(q, want, sm)
+    got = qc.clone().to(dev)
+    store_query_cache(q.to(dev), got, sm.to(dev))
+    assert torch.equal(got.cpu(), want)
+    # empty slot mapping and empty cache are no-ops
+    store_query_cache(q.to(dev), got, sm[:0].to(dev))
+    store_query_cache(q.to(dev), got[:0], sm.to(dev))
+    assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("style", ["aliased", "cow"])
+def test_compress_kv_bit_exact(dev, dtype, style):
+    from zipage_amd.kernel import compress_kv
+    s = _setup(11, dtype, L=2, B=4, Hkv=3, Hq=3, nb_choices=(3, 4, 5), budget=2, num_pages=40)
+    k, v, enc = s["k"], s["v"], s["enc"]
+    L, _, BS, Hkv, D = k.shape
+    B, NB = enc.shape
+    g = torch.Generator().manual_seed(5)
+    scores = torch.rand((L, B, Hkv, NB * BS), generator=g)
+    scores = O.pad_mask(scores.view(L, B, Hkv, NB, BS), enc).view(L, B, Hkv, NB * BS)
+    flag = O.topk_mask(scores, 2 * BS).view(L, B, Hkv, NB, BS)
+    if style == "aliased":   # already-compressed sequences: target = own first pages
+        target = s["target"]
+    else:                    # copy-on-write: two fresh pages then own pages
+        used = cases.touched_pages(enc)
+        fresh = [p for p in range(40) if p not in used]
+        target = torch.tensor([[fresh[2 * b], fresh[2 * b + 1], t[2]] for b, t in enumerate(s["tables"])],
+                              dtype=torch.int32)
+    wk, wv = k.clone(), v.clone()
+    O.compress_kv_loop(wk, wv, flag, enc, target)
+    gk, gv = k.clone().to(dev), v.clone().to(dev)
+    compress_kv(gk, gv, flag.to(dev), enc.to(dev), target.to(dev))
+    assert torch.equal(gk.cpu().view(torch.uint8), wk.view(torch.uint8))
+    assert torch.equal(gv.cpu().view(torch.uint8), wv.view(torch.uint8))
+
+
+def test_compress_kv_strided_views(dev):
+    """key/value as slices of one (2, L, pages, BS, Hkv, D) allocation, layer-sliced."""
+    from zipage_amd.kernel import compress_kv
+    dtype = torch.bfloat16
+    s = _setup(12, dtype, L=3, B=2, Hkv=2, Hq=2, nb_choices=(3,), budget=2, num_pages=10)
+    kv = torch.stack([s["k"], s["v"]])
+    enc, target = s["enc"], s["target"]
+    L, BS, Hkv = 2, 256, 2
+    g = torch.Generator().manual_seed(6)
+    flag = O.topk_mask(torch.rand((L, 2, Hkv, 3 * BS), generator=g), 2 * BS).view(L, 2, Hkv, 3, BS)
+    want = kv.clone()
+    O.compress_kv_loop(want[0, 1:3], want[1, 1:3], flag, enc, target)
+    got = kv.clone().to(dev)
+    compress_kv(got[0, 1:3], got[1, 1:3], flag.to(dev), enc.to(dev), target.to(dev))
+    assert torch.equal(got.cpu().view(torch.uint8), want.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_compress_score_bit_exact(dev, dtype):
+    from zipage_amd.kernel import compress_score
+    s = _setup(13, dtype, L=2, B=3, Hkv=4, Hq=4, nb_choices=(3, 4), budget=2, num_pages=30,
+               score_cache=True)
+    enc, target, sc = s["enc"], s["target"], s["sc"]
+    L, _, BS, Hkv = sc.shape
+    B, NB = enc.shape
+    g = torch.Generator().manual_seed(7)
+    scores = O.pad_mask(torch.rand((L, B, Hkv, NB, BS), generator=g), enc)
+    flag = O.topk_mask(scores.view(L, B, Hkv, NB * BS), 2 * BS).view(L, B, Hkv, NB, BS)
+    want = O.compress_score(sc.clone(), flag, enc, target)
+    got = compress_score(sc.clone().to(dev), flag.to(dev), enc.to(dev), target.to(dev))
+    assert torch.equal(got.cpu().view(torch.uint8), want.view(torch.uint8))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_topk_mask_ties_lowest_index(dev, dtype):
+    from zipage_amd.kernel import topk_mask
+    g = torch.Generator().manual_seed(17)
+    rows, T = 24, 2304
+    # few distinct values -> massive ties; sprinkle +-inf, zeros of both signs
+    x = (torch.randint(0, 40, (rows, T), generator=g).float() / 64.0 - 0.25).to(dtype)
+    x[0, :100] = float("inf")
+    x[1, 5:300] = float("-inf")
+    x[2, ::2] = 0.0
+    x[2, 1::2] = -0.0
+    x[3] = 0.125
+    for k in (2048, 1, T, 0, 777):
+        want = O.topk_mask(x, k)
+        got = topk_mask(x.to(dev), k).cpu()
+        assert got.dtype == torch.bool
+        assert torch.equal(got, want), f"k={k}"
+        assert (got.sum(-1) == k).all()
+    y = torch.randn((3, 2, 5, 1280), generator=g).to(dtype)
+    assert torch.equal(topk_mask(y.to(dev), 1024).cpu(), O.topk_mask(y, 1024))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("method", ["max", "sum"])
+def test_global_score(dev, dtype, method):
+    from zipage_amd.kernel import global_score
+    s = _setup(19, dtype, L=2, B=3, Hkv=4, Hq=4, nb_choices=(2, 3), budget=2, num_pages=16,
+               score_cache=True)
+    enc, sc = s["enc"], s["sc"]
+    L, _, BS, Hkv = sc.shape
+    B, NB = enc.shape
+    g = torch.Generator().manual_seed(23)
+    scores = torch.rand((L, B, Hkv, NB, BS), generator=g).to(dtype)
+    compressed = torch.tensor([True, False, True])
+    ws, wc = scores.clone(), sc.clone()
+    O.global_score(ws, wc, enc, compressed, 0.9, method)
+    gs, gc = scores.clone().to(dev), sc.clone().to(dev)
+    out = global_score(gs, gc, enc.to(dev), compressed.to(dev), 0.9, method)
+    assert out.data_ptr() == gs.data_ptr()
+    if method == "max" or dtype == torch.float32:
+        assert torch.equal(gs.cpu(), ws) and torch.equal(gc.cpu(), wc)
+    else:
+        _ulp_close(gs, ws, dtype)
+        _ulp_close(gc, wc, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("continues", [False, True])
+def test_pool_scores(dev, dtype, continues):
+    from zipage_amd.kernel import pool_scores
+    g = torch.Generator().manual_seed(29)
+    L, B, Hkv, NB, BS = 2, 3, 2, 3, 256
+    scores = torch.rand((L, B, Hkv, NB, BS), generator=g).to(dtype)
+    compressed = torch.tensor([False, True, False])
+    for ksz in (5, 7, 1):
+        want = O.pool_scores(scores, compressed, ksz, continues)
+        got = pool_scores(scores.to(dev), compressed.to(dev), ksz, continues)
+        assert torch.equal(got.cpu(), want)
+    want = O.pool_scores(scores, compressed, 7, continues, mode="avg")
+    got = pool_scores(scores.to(dev), compressed.to(dev), 7, continues, mode="avg")
+    _ulp_close(got, want, dtype)
+    # all compressed and not continues -> untouched
+    allc = torch.tensor([True, True, True])
+    assert torch.equal(pool_scores(scores.to(dev), allc.to(dev), 5, False).cpu(),
+                       O.pool_scores(scores, allc, 5, False))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_window_mask_and_epilogue(dev, dtype):
+    from zipage_amd.kernel import window_mask, score_epilogue
+    enc = torch.tensor(cases.REF_TABLES["attention"], dtype=torch.int32)
+    g = torch.Generator().manual_seed(31)
+    L, B, Hkv, NB, BS = 2, 2, 3, 4, 256
+    scores = torch.rand((L, B, Hkv, NB, BS), generator=g).to(dtype)
+    red = torch.rand((L, B, Hkv, NB, BS), generator=g).to(dtype)
+    want = O.window_mask(scores.clone(), enc, 24)
+    got = window_mask(scores.clone().to(dev), enc.to(dev), 24)
+    assert torch.equal(got.cpu(), want)
+    # full epilogue in the runner's order
+    w = O.max_normalise(scores.clone())
+    w = O.combine_scores(w, O.max_normalise(red.clone()), 0.2)
+    w = O.attention_sink(w.contiguous(), 4)
+    w = O.window_mask(w, enc, 16)
+    w = O.pad_mask(w, enc)
+    g2 = score_epilogue(scores.clone().to(dev), enc.to(dev), red.to(dev), max_norm_scores=True,
+                        max_norm_red=True, redudancy_lambda=0.2, sink_len=4, window=16,
+                        mask_pad=True)
+    assert torch.equal(g2.cpu(), w)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_key_norm(dev, dtype):
+    from zipage_amd.kernel import key_norm
+    s = _setup(37, dtype, L=2, B=2, Hkv=3, Hq=3, nb_choices=(2, 3), budget=2, num_pages=12)
+    s["k"][0, s["tables"][0][0], 5, 1] = 0  # a zero key clamps to eps
+    want = O.key_norm(s["k"], s["enc"])
+    got = key_norm(s["k"].to(dev), s["enc"].to(dev))
+    if dtype == torch.float32:
+        _rel_close(got, want, rel=1e-6)
+    else:
+        _ulp_close(got, want, dtype, frac_exact=0.999)
+
+
+# ------------------------------------------------------------------ scorer
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cfg", [dict(Hkv=2, Hq=8, W=32), dict(Hkv=2, Hq=4, W=32),
+                                 dict(Hkv=2, Hq=16, W=24), dict(Hkv=3, Hq=3, W=16),
+                                 dict(Hkv=1, Hq=7, W=16)])
+@pytest.mark.parametrize("reduced", ["mean", "max"])
+def test_attention_score(dev, dtype, cfg, reduced):
+    from zipage_amd.kernel import attention_score
+    if reduced == "max" and cfg["Hq"] not in (8, 16):
+        pytest.skip("max reduction covered on two shapes")
+    s = _setup(41, dtype, L=2, B=3, nb_choices=(2, 3, 4), num_pages=20, **cfg)
+    args = (s["k"], s["q"], s["seq_idx"], s["enc"])
+    want, wlog = O.attention_score(*args, reduced=reduced, return_logits=True)
+    got, glog = attention_score(*(a.to(dev) for a in args), reduced=reduced, return_logits=True)
+    assert got.shape == want.shape and got.dtype == dtype
+    assert glog.shape == wlog.shape
+    if dtype == torch.float32:
+        _rel_close(glog, wlog, rel=1e-4, abs_floor=1e-5)
+        _rel_close(got, want, rel=1e-3, abs_floor=1e-9)
+    else:
+        _ulp_close(glog, wlog, dtype, ulps=1, frac_exact=0.995)
+        _ulp_close(got, want, dtype, ulps=2, frac_exact=0.9)
+    # without logits the scores are the same bits
+    got2 = attention_score(*(a.to(dev) for a in args), reduced=reduced)
+    assert torch.equal(got2, got)
+
+
+def test_attention_score_reference_script_shape(dev):
+    """Shape of the reference's own script: 2 seqs, tables [[0,1,2,-5],[5,6,-9,-1]], W=24,
+    Hq=16, Hkv=2, D=128, fp16 (tests/test_attention_score.py:314-358)."""
+    from zipage_amd.kernel import attention_score
+    dtype = torch.float16
+    enc = torch.tensor(cases.REF_TABLES["attention"], dtype=torch.int32)
+    k, _, q, _ = cases.make_caches(43, 4, 16, 256, 2, 16, 128, 24, 8, dtype, with_v=False)
+    seq_idx = torch.tensor([3, 6], dtype=torch.int32)
+    want = O.attention_score(k, q, seq_idx, enc)
+    got = attention_score(k.to(dev), q.to(dev), seq_idx.to(dev), enc.to(dev))
+    _ulp_close(got, want, dtype, ulps=2, frac_exact=0.9)
+    assert (got.cpu()[1, 1, :, 3] == 0).all()  # pad page scores exactly 0
+
+
+# ------------------------------------------------------------------ redundancy
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("thr", [0.5, 0.0, 0.1])
+def test_lightning_redundancy(dev, dtype, thr):
+    from zipage_amd.kernel import lightning_redudancy_score
+    s = _setup(47, dtype, L=2, B=2, Hkv=2, Hq=2, nb_choices=(2, 3), num_pages=12)
+    k = s["k"]
+    # correlated keys so that similarities exceed the threshold
+    base = torch.randn((1, 1, 1, 2, 128), generator=torch.Generator().manual_seed(1))
+    k = (k.float() * 0.6 + base).to(dtype)
+    wl, wr = O.lightning_redudancy_score(k, s["enc"], threshold=thr, temperature=0.4,
+                                         return_logits=True)
+    gl, gr = lightning_redudancy_score(k.to(dev), s["enc"].to(dev), threshold=thr, temperature=0.4,
+                                       return_logits=True)
+    if dtype == torch.float32:
+        _rel_close(gl, wl, rel=1e-4, abs_floor=1e-3)
+        _rel_close(gr, wr, rel=1e-3, abs_floor=1e-9)
+    else:
+        _ulp_close(gl, wl, dtype, ulps=1, frac_exact=0.97)
+        _ulp_close(gr, wr, dtype, ulps=2, frac_exact=0.9)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_raw_redundancy(dev, dtype):
+    from zipage_amd.kernel import raw_redudancy_score
+    s = _setup(53, dtype, L=1, B=2, Hkv=2, Hq=2, nb_choices=(2, 3), num_pages=12)
+    base = torch.randn((1, 1, 1, 2, 128), generator=torch.Generator().manual_seed(2))
+    k = (s["k"].float() * 0.6 + base).to(dtype)
+    mode = "reference" if dtype == torch.float32 else "fp32"
+    wl, wr = O.raw_redudancy_score(k, s["enc"], threshold=0.5, temperature=0.4,
+                                   return_logits=True, rounding=mode)
+    gl, gr = raw_redudancy_score(k.to(dev), s["enc"].to(dev), threshold=0.5, temperature=0.4,
+                                 return_logits=True)
+    if dtype == torch.float32:
+        _rel_close(gl, wl, rel=1e-4, abs_floor=1e-2)
+        _rel_close(gr, wr, rel=1e-3, abs_floor=1e-9)
+    else:
+        _ulp_close(gl, wl, dtype, ulps=1)
+        _ulp_close(gr, wr, dtype, ulps=4)

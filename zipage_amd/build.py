@@ -1,0 +1,46 @@
+"""Build libzipage_hip.so (gfx950) in-tree with hipcc.
+
+Run as ``python -m zipage_amd.build``.  The library is one shared object with a plain C
+ABI (``include/zipage_hip.h``); it does not link against torch.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libzipage_hip.so")
+
+# packed fp32 VALU ops are disabled on purpose (some forms misbehave on this fleet)
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def sources():
+    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def build(verbose: bool = True) -> str:
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    cmd = [hipcc, *FLAGS, *sources(), "-o", LIB + ".tmp"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in proc.stderr.splitlines()
+                    if "is not a recognized feature for this target" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{proc.stdout}\n{err}")
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+    os.replace(LIB + ".tmp", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build())

@@ -1,0 +1,112 @@
+// Shared device/host helpers for the KV-compression kernels (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#include "../../include/zipage_hip.h"
+
+#define ZP_WAVE 64
+
+// ---------------------------------------------------------------- error reporting
+void zp_set_error(const char* fmt, ...);
+
+#define ZP_REQUIRE(cond, ...)            \
+  do {                                   \
+    if (!(cond)) {                       \
+      zp_set_error(__VA_ARGS__);         \
+      return ZP_EINVAL;                  \
+    }                                    \
+  } while (0)
+
+#define ZP_LAUNCH_CHECK()                                              \
+  do {                                                                 \
+    hipError_t e_ = hipGetLastError();                                 \
+    if (e_ != hipSuccess) {                                            \
+      zp_set_error("%s:%d HIP launch failed: %s", __FILE__, __LINE__,  \
+                   hipGetErrorString(e_));                             \
+      return ZP_EHIP;                                                  \
+    }                                                                  \
+  } while (0)
+
+// ---------------------------------------------------------------- element types
+// Storage element tags.  bf16/fp16 are kept as raw 16-bit patterns in memory.
+struct BF16 { typedef uint16_t raw; static constexpr int bytes = 2; };
+struct F16  { typedef uint16_t raw; static constexpr int bytes = 2; };
+struct F32  { typedef float raw;    static constexpr int bytes = 4; };
+
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t h) {
+  return __uint_as_float(((uint32_t)h) << 16);
+}
+// Round-to-nearest-even, infinities preserved, NaN kept quiet.
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+__device__ __forceinline__ float f16_bits_to_float(uint16_t h) {
+  union { uint16_t u; _Float16 f; } c; c.u = h; return (float)c.f;
+}
+__device__ __forceinline__ uint16_t float_to_f16_bits(float f) {
+  union { uint16_t u; _Float16 f; } c; c.f = (_Float16)f; return c.u;
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<BF16> {
+  __device__ static __forceinline__ float ld(const void* p, int64_t i) { return bf16_bits_to_float(((const uint16_t*)p)[i]); }
+  __device__ static __forceinline__ void st(void* p, int64_t i, float v) { ((uint16_t*)p)[i] = float_to_bf16_bits(v); }
+  __device__ static __forceinline__ float rnd(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }
+};
+template <> struct Elem<F16> {
+  __device__ static __forceinline__ float ld(const void* p, int64_t i) { return f16_bits_to_float(((const uint16_t*)p)[i]); }
+  __device__ static __forceinline__ void st(void* p, int64_t i, float v) { ((uint16_t*)p)[i] = float_to_f16_bits(v); }
+  __device__ static __forceinline__ float rnd(float v) { return f16_bits_to_float(float_to_f16_bits(v)); }
+};
+template <> struct Elem<F32> {
+  __device__ static __forceinline__ float ld(const void* p, int64_t i) { return ((const float*)p)[i]; }
+  __device__ static __forceinline__ void st(void* p, int64_t i, float v) { ((float*)p)[i] = v; }
+  __device__ static __forceinline__ float rnd(float v) { return v; }
+};
+
+// Dispatch a templated launcher on the runtime dtype tag.
+#define ZP_DISPATCH_DTYPE(dtype, ...)                                   \
+  switch (dtype) {                                                      \
+    case ZP_BF16: { typedef BF16 T; __VA_ARGS__; } break;               \
+    case ZP_F16:  { typedef F16 T;  __VA_ARGS__; } break;               \
+    case ZP_F32:  { typedef F32 T;  __VA_ARGS__; } break;               \
+    default: zp_set_error("unknown dtype tag %d", (int)(dtype)); return ZP_EINVAL; \
+  }
+
+static inline int zp_dtype_bytes(int dtype) { return dtype == ZP_F32 ? 4 : 2; }
+
+// ---------------------------------------------------------------- page-table codes
+// id >= 0: full page; -1: padding; x < -1: the sequence's last page, id = -x-2.
+__device__ __forceinline__ bool page_is_pad(int code) { return code == -1; }
+__device__ __forceinline__ bool page_is_last(int code) { return code < -1; }
+__device__ __forceinline__ int page_id(int code) { return code < -1 ? -code - 2 : code; }
+
+// ---------------------------------------------------------------- wave helpers
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ int wave_sum_i(int v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
+__device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
+__device__ __forceinline__ uint64_t lanemask_lt() {
+  return (1ull << lane_id()) - 1ull;
+}
+
+struct __attribute__((aligned(16))) vec16 { uint32_t x, y, z, w; };

@@ -1,0 +1,468 @@
+// Key-redundancy scores: cosine-similarity Gram matrix of cached keys, per page
+// ("lightning") or over the whole sequence ("raw"), with the reference's claim rule:
+// the diagonal is zeroed and, for every column, the LAST row whose similarity exceeds the
+// threshold is zeroed too; the row sums are the redundancy logits.
+//
+// The Gram matrix is symmetric, so "last row over the threshold in column j" equals "last
+// column over the threshold in row j".  A wave owns 32 rows for all columns, tracks per
+// row the plain row sum and the last column over the threshold (with its value); the
+// claimed entries are subtracted afterwards from the rows they belong to:
+//     r_i = sum_j S_ij  -  sum_{j : c*(j) = i} S_ji .
+// This needs one pass over the columns and no cross-wave ordering.
+//
+// Arithmetic follows the reference: keys are divided by their cache-dtype norm in fp32 and
+// the dot products are fp32 (v_mfma_f32_32x32x2_f32, A = 32 key rows in registers,
+// B = 64-key column tiles normalised on the way into double-buffered LDS).
+#include "common.h"
+#include <math.h>
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr int kDmax = 128;
+constexpr int TN = 64;                  // keys per column tile
+constexpr int ROWF = kDmax + 2;         // floats per LDS row (bank-conflict-free pad)
+constexpr int KS = kDmax / 2;           // MFMA k-steps (2 per instruction)
+
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+template <typename T> struct Unpack;
+template <> struct Unpack<F32> {
+  static constexpr int N = 4;
+  __device__ static __forceinline__ void run(const vec16& v, float* o) {
+    o[0] = __uint_as_float(v.x); o[1] = __uint_as_float(v.y);
+    o[2] = __uint_as_float(v.z); o[3] = __uint_as_float(v.w);
+  }
+};
+template <> struct Unpack<BF16> {
+  static constexpr int N = 8;
+  __device__ static __forceinline__ void run(const vec16& v, float* o) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      o[2 * i] = __uint_as_float(w[i] << 16);
+      o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+};
+template <> struct Unpack<F16> {
+  static constexpr int N = 8;
+  __device__ static __forceinline__ void run(const vec16& v, float* o) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      o[2 * i] = f16_bits_to_float((uint16_t)(w[i] & 0xffffu));
+      o[2 * i + 1] = f16_bits_to_float((uint16_t)(w[i] >> 16));
+    }
+  }
+};
+
+struct GramArgs {
+  const char* k;
+  const int32_t* table;
+  void* r_out;     // lightning: (rows, NB*BS) row sums in the cache dtype
+  float* ws_sum;   // raw: fp32 plain row sums
+  int32_t* ws_col; // raw: last column over the threshold (logical index, -1 none)
+  float* ws_val;   // raw: its value
+  int B, NB, BS, Hkv, D, num_pages;
+  int64_t k_sl, k_sp;
+  float threshold, eps;
+};
+
+template <typename T, bool RAW>
+__global__ __launch_bounds__(kThreads) void gram_kernel(GramArgs p) {
+  constexpr int NE = Unpack<T>::N;                  // elements per 16-byte piece
+  constexpr int PIECES = kDmax / NE;                // pieces per full key row
+  constexpr int ROWS_PER_IT = kThreads / PIECES;
+  constexpr int STAGE_IT = TN / ROWS_PER_IT;
+  constexpr int NSUB = TN / 32;
+
+  extern __shared__ __align__(16) char smem[];
+  float* kbuf0 = (float*)smem;
+  float* kbuf1 = kbuf0 + TN * ROWF;
+  float* l_sum = kbuf1 + TN * ROWF;                 // lightning: [BS] row sums
+  float* l_val = l_sum + (RAW ? 0 : p.BS);          //            [BS] claimed values
+  int* l_col = (int*)(l_val + (RAW ? 0 : p.BS));    //            [BS] claimed columns
+  int* vpage = l_col + (RAW ? 0 : p.BS);            // [NB] valid page ids (raw)
+  int* vidx = vpage + p.NB;                         // [NB] their table index
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const int jp = blockIdx.x % p.NB;                 // row page (table index)
+  const int h = (blockIdx.x / p.NB) % p.Hkv;
+  const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
+  const int l = blockIdx.x / (p.NB * p.Hkv * p.B);
+  const int Tn = p.NB * p.BS;
+  const int64_t orow = (((int64_t)l * p.B + b) * p.Hkv + h);
+  const float epsr = Elem<T>::rnd(p.eps);
+
+  const int code = p.table[(int64_t)b * p.NB + jp];
+  int rpid = page_is_pad(code) ? -1 : page_id(code);
+  if (rpid >= p.num_pages) rpid = -1;
+  if (rpid < 0) {  // pad page: logits -inf (lightning); raw marks it in the epilogue
+    if (!RAW)
+      for (int s = tid; s < p.BS; s += kThreads)
+        Elem<T>::st(p.r_out, orow * Tn + (int64_t)jp * p.BS + s, -INFINITY);
+    return;
+  }
+
+  __shared__ int ncols_s;
+  if (tid == 0) {
+    int n = 0;
+    if (RAW) {
+      for (int j = 0; j < p.NB; ++j) {
+        const int c = p.table[(int64_t)b * p.NB + j];
+        const int pid = page_is_pad(c) ? -1 : page_id(c);
+        if (pid >= 0 && pid < p.num_pages) { vpage[n] = pid; vidx[n] = j; ++n; }
+      }
+    } else {
+      vpage[0] = rpid; vidx[0] = jp; n = 1;
+    }
+    ncols_s = n;
+  }
+  for (int i = tid; i < 2 * TN * ROWF; i += kThreads) kbuf0[i] = 0.f;
+  __syncthreads();
+  const int tiles_per_page = p.BS / TN;
+  const int ntiles = ncols_s * tiles_per_page;
+  const int dpieces = p.D / NE;
+  const int64_t k_row = (int64_t)p.Hkv * p.D * T::bytes;
+  const char* kbase = p.k + (l * p.k_sl) * T::bytes + (int64_t)h * p.D * T::bytes;
+
+  const int st_piece = tid % PIECES, st_row0 = tid / PIECES;
+  vec16 pre[STAGE_IT];
+  auto issue_loads = [&](int tile) {
+    const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
+    const char* src = kbase + (int64_t)vpage[vp] * p.k_sp * T::bytes + (int64_t)toff * k_row;
+#pragma unroll
+    for (int i = 0; i < STAGE_IT; ++i) {
+      const int row = st_row0 + i * ROWS_PER_IT;
+      pre[i] = vec16{0u, 0u, 0u, 0u};
+      if (st_piece < dpieces) pre[i] = *(const vec16*)(src + (int64_t)row * k_row + st_piece * 16);
+    }
+  };
+  // normalise (k / max(rnd(|k|), rnd(eps)) in fp32) on the way into LDS
+  auto commit_loads = [&](float* buf) {
+#pragma unroll
+    for (int i = 0; i < STAGE_IT; ++i) {
+      const int row = st_row0 + i * ROWS_PER_IT;
+      float e[NE];
+      Unpack<T>::run(pre[i], e);
+      float ss = 0.f;
+#pragma unroll
+      for (int q = 0; q < NE; ++q) ss += e[q] * e[q];
+#pragma unroll
+      for (int o = PIECES >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      const float n = fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
+      if (st_piece < dpieces) {
+        float* d = buf + row * ROWF + st_piece * NE;
+#pragma unroll
+        for (int q = 0; q < NE; q += 2) *(float2*)(d + q) = make_float2(e[q] / n, e[q + 1] / n);
+      }
+    }
+  };
+
+  const int row_blocks = p.BS / 32;
+  const int NR = (row_blocks + kWaves - 1) / kWaves;
+  for (int rr = 0; rr < NR; ++rr) {
+    const int rb = rr * kWaves + wave;
+    const bool active = rb < row_blocks;
+    // ---- A fragments: this lane's key row, normalised; element k = 2s + half
+    float afrag[KS];
+    {
+      const int slot = (active ? rb : 0) * 32 + col;
+      const char* src = kbase + (int64_t)rpid * p.k_sp * T::bytes + (int64_t)slot * k_row;
+      float ss = 0.f;
+#pragma unroll
+      for (int pc = 0; pc < PIECES; ++pc) {
+        float e[NE];
+        vec16 v = vec16{0u, 0u, 0u, 0u};
+        if (pc < dpieces) v = *(const vec16*)(src + pc * 16);
+        Unpack<T>::run(v, e);
+#pragma unroll
+        for (int q = 0; q < NE; ++q) ss += e[q] * e[q];
+#pragma unroll
+        for (int q = 0; q < NE / 2; ++q) afrag[pc * (NE / 2) + q] = half ? e[2 * q + 1] : e[2 * q];
+      }
+      const float n = fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
+#pragma unroll
+      for (int s = 0; s < KS; ++s) afrag[s] = active ? afrag[s] / n : 0.f;
+    }
+    float rsum[16], cval[16];
+    int ccol[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { rsum[r] = 0.f; cval[r] = 0.f; ccol[r] = -1; }
+
+    if (ntiles > 0) { issue_loads(0); commit_loads(kbuf0); }
+    __syncthreads();
+    for (int tile = 0; tile < ntiles; ++tile) {
+      float* cur = (tile & 1) ? kbuf1 : kbuf0;
+      float* nxt = (tile & 1) ? kbuf0 : kbuf1;
+      if (tile + 1 < ntiles) issue_loads(tile + 1);
+      const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
+      const int jc = vidx[vp];
+      if (active) {
+#pragma unroll
+        for (int st = 0; st < NSUB; ++st) {
+          f32x16_t acc;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+          const float* brow = cur + (st * 32 + col) * ROWF + half;
+#pragma unroll
+          for (int s = 0; s < KS; ++s)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[s], brow[2 * s], acc, 0, 0, 0);
+          const int cslot = toff + st * 32 + col;
+          const int cidx = jc * p.BS + cslot;  // logical column index of this lane
+          const bool same_page = jc == jp;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+            float s = acc[r];
+            if (same_page && rslot == cslot) s = 0.f;
+            rsum[r] += s;
+            if (s > p.threshold) { ccol[r] = cidx; cval[r] = s; }
+          }
+        }
+      }
+      if (tile + 1 < ntiles) commit_loads(nxt);
+      __syncthreads();
+    }
+    // ---- combine over the 32 lanes of each half (they share rows)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float s = rsum[r];
+      int c = ccol[r];
+      float v = cval[r];
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) {
+        s += __shfl_xor(s, o, 64);
+        const int oc = __shfl_xor(c, o, 64);
+        const float ov = __shfl_xor(v, o, 64);
+        if (oc > c) { c = oc; v = ov; }
+      }
+      if (active && col == 0) {
+        const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+        if (RAW) {
+          const int64_t oi = orow * Tn + (int64_t)jp * p.BS + rslot;
+          p.ws_sum[oi] = s;
+          p.ws_col[oi] = c;
+          p.ws_val[oi] = v;
+        } else {
+          l_sum[rslot] = s;
+          l_col[rslot] = c - jp * p.BS;  // column slot inside the page (or negative)
+          l_val[rslot] = v;
+        }
+      }
+    }
+  }
+  if (!RAW) {
+    __syncthreads();
+    for (int i = tid; i < p.BS; i += kThreads) {
+      float corr = 0.f;
+      for (int j = 0; j < p.BS; ++j)
+        if (l_col[j] == i) corr += l_val[j];
+      Elem<T>::st(p.r_out, orow * Tn + (int64_t)jp * p.BS + i, l_sum[i] - corr);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ softmax epilogue
+// One workgroup per (layer, sequence, head) row of T logits:
+//   raw only: r_i = rowsum_i - sum_{j: c*(j)=i} v_j, pad pages -inf
+//   x = rnd(r / divisor); x = rnd(x - max); out = rnd(exp(x) / sum)
+__device__ __forceinline__ float block_reduce(float v, float* lds, bool is_max) {
+  if (is_max) v = wave_max(v); else v = wave_sum(v);
+  __syncthreads();
+  if (lane_id() == 0) lds[wave_id()] = v;
+  __syncthreads();
+  float m = lds[0];
+#pragma unroll
+  for (int i = 1; i < kWaves; ++i) m = is_max ? fmaxf(m, lds[i]) : m + lds[i];
+  return m;
+}
+
+template <typename T, bool RAW>
+__global__ __launch_bounds__(kThreads) void red_softmax_kernel(
+    void* __restrict__ red, void* __restrict__ logits, const int32_t* __restrict__ table,
+    const float* __restrict__ ws_sum, const int32_t* __restrict__ ws_col,
+    const float* __restrict__ ws_val, int B, int NB, int BS, int Hkv, int num_pages,
+    float tscale /* raw: temperature; lightning: temperature*BS */) {
+  extern __shared__ __align__(16) char smem[];
+  __shared__ float red_lds[kWaves];
+  const int Tn = NB * BS;
+  float* x = (float*)smem;          // [Tn]
+  int* ccol = (int*)(x + Tn);       // [Tn] raw only
+  float* cval = (float*)(ccol + (RAW ? Tn : 0));
+  const int64_t row = blockIdx.x;
+  const int b = (int)((row / Hkv) % B);
+  const int64_t base = row * Tn;
+  const int32_t* trow = table + (int64_t)b * NB;
+  int nvalid = 0;
+  for (int j = 0; j < NB; ++j) {
+    const int c = trow[j];
+    const int pid = page_is_pad(c) ? -1 : page_id(c);
+    nvalid += (pid >= 0 && pid < num_pages) ? 1 : 0;
+  }
+  const float divisor = RAW ? tscale * (float)(nvalid * BS) : tscale;
+  if (RAW) {
+    for (int t = threadIdx.x; t < Tn; t += kThreads) {
+      const int c = trow[t / BS];
+      const int pid = page_is_pad(c) ? -1 : page_id(c);
+      const bool ok = pid >= 0 && pid < num_pages;
+      ccol[t] = ok ? ws_col[base + t] : -1;
+      cval[t] = ok ? ws_val[base + t] : 0.f;
+    }
+    __syncthreads();
+  }
+  float mloc = -INFINITY;
+  for (int t = threadIdx.x; t < Tn; t += kThreads) {
+    float r;
+    if (RAW) {
+      const int c = trow[t / BS];
+      const int pid = page_is_pad(c) ? -1 : page_id(c);
+      if (pid >= 0 && pid < num_pages) {
+        float corr = 0.f;
+        for (int j = 0; j < Tn; ++j)
+          if (ccol[j] == t) corr += cval[j];
+        r = Elem<T>::rnd(ws_sum[base + t] - corr);
+      } else {
+        r = -INFINITY;
+      }
+    } else {
+      r = Elem<T>::ld(red, base + t);
+    }
+    if (logits) Elem<T>::st(logits, base + t, r);
+    const float xv = Elem<T>::rnd(r / divisor);
+    x[t] = xv;
+    mloc = fmaxf(mloc, xv);
+  }
+  const float m = block_reduce(mloc, red_lds, true);
+  float sloc = 0.f;
+  for (int t = threadIdx.x; t < Tn; t += kThreads) {
+    const float e = expf(Elem<T>::rnd(x[t] - m));
+    x[t] = e;
+    sloc += e;
+  }
+  const float ssum = block_reduce(sloc, red_lds, false);
+  for (int t = threadIdx.x; t < Tn; t += kThreads) Elem<T>::st(red, base + t, x[t] / ssum);
+}
+
+int check_common(const char* name, const void* k_cache, const int32_t* table, void* red_out,
+                 int L, int B, int NB, int BS, int Hkv, int D, int dtype, int64_t k_sl,
+                 int64_t k_sp) {
+  ZP_REQUIRE(k_cache && table && red_out, "%s: null pointer", name);
+  ZP_REQUIRE(L >= 0 && B >= 0 && NB > 0 && BS > 0 && Hkv > 0 && D > 0, "%s: bad dims", name);
+  ZP_REQUIRE(dtype >= ZP_BF16 && dtype <= ZP_F32, "%s: unknown dtype tag %d", name, dtype);
+  const int es = zp_dtype_bytes(dtype);
+  if (!(D <= kDmax && (D * es) % 16 == 0)) {
+    zp_set_error("%s: head_dim %d unsupported (need <= %d and a multiple of %d)", name, D, kDmax,
+                 16 / es);
+    return ZP_EUNSUPPORTED;
+  }
+  if (BS % TN != 0) {
+    zp_set_error("%s: page size %d is not a multiple of %d", name, BS, TN);
+    return ZP_EUNSUPPORTED;
+  }
+  ZP_REQUIRE(((uintptr_t)k_cache % 16) == 0 && (k_sl * es) % 16 == 0 && (k_sp * es) % 16 == 0,
+             "%s: key cache must be 16-byte aligned", name);
+  return ZP_OK;
+}
+
+template <typename T, bool RAW>
+int launch_gram(const GramArgs& a, int L, hipStream_t st) {
+  const size_t smem = sizeof(float) * 2 * TN * ROWF + (RAW ? 0 : (size_t)a.BS * 12) +
+                      sizeof(int) * 2 * a.NB;
+  if (smem > 64 * 1024 &&
+      hipFuncSetAttribute((const void*)gram_kernel<T, RAW>,
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+    zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
+    return ZP_EHIP;
+  }
+  dim3 grid((unsigned)((int64_t)L * a.B * a.Hkv * a.NB));
+  hipLaunchKernelGGL((gram_kernel<T, RAW>), grid, dim3(kThreads), smem, st, a);
+  ZP_LAUNCH_CHECK();
+  return ZP_OK;
+}
+
+template <typename T, bool RAW>
+int launch_softmax(void* red, void* logits, const int32_t* table, const float* ws_sum,
+                   const int32_t* ws_col, const float* ws_val, int L, int B, int NB, int BS,
+                   int Hkv, int num_pages, double temperature, hipStream_t st) {
+  const size_t smem = (size_t)NB * BS * (RAW ? 12 : 4);
+  if (smem > 150 * 1024) {
+    zp_set_error("redundancy: a row of %d tokens exceeds LDS", NB * BS);
+    return ZP_EUNSUPPORTED;
+  }
+  if (smem > 64 * 1024 &&
+      hipFuncSetAttribute((const void*)red_softmax_kernel<T, RAW>,
+                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+    zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
+    return ZP_EHIP;
+  }
+  dim3 grid((unsigned)((int64_t)L * B * Hkv));
+  hipLaunchKernelGGL((red_softmax_kernel<T, RAW>), grid, dim3(kThreads), smem, st, red, logits,
+                     table, ws_sum, ws_col, ws_val, B, NB, BS, Hkv, num_pages,
+                     RAW ? (float)temperature : (float)(temperature * (double)BS));
+  ZP_LAUNCH_CHECK();
+  return ZP_OK;
+}
+
+}  // namespace
+
+extern "C" int zp_redundancy_lightning(const void* k_cache, const int32_t* block_table,
+                                       void* red_out, void* logits_out, int32_t L, int32_t B,
+                                       int32_t NB, int32_t BS, int32_t Hkv, int32_t D,
+                                       int32_t num_pages, int64_t k_sl, int64_t k_sp,
+                                       float threshold, double temperature, int32_t dtype,
+                                       void* stream) {
+  int rc = check_common("redundancy_lightning", k_cache, block_table, red_out, L, B, NB, BS, Hkv,
+                        D, dtype, k_sl, k_sp);
+  if (rc != ZP_OK) return rc;
+  if (L == 0 || B == 0) return ZP_OK;
+  GramArgs a;
+  a.k = (const char*)k_cache; a.table = block_table; a.r_out = red_out;
+  a.ws_sum = nullptr; a.ws_col = nullptr; a.ws_val = nullptr;
+  a.B = B; a.NB = NB; a.BS = BS; a.Hkv = Hkv; a.D = D; a.num_pages = num_pages;
+  a.k_sl = k_sl; a.k_sp = k_sp; a.threshold = threshold; a.eps = 1e-6f;
+  hipStream_t st = (hipStream_t)stream;
+  ZP_DISPATCH_DTYPE(dtype, {
+    rc = launch_gram<T, false>(a, L, st);
+    if (rc != ZP_OK) return rc;
+    rc = launch_softmax<T, false>(red_out, logits_out, block_table, nullptr, nullptr, nullptr, L,
+                                  B, NB, BS, Hkv, num_pages, temperature, st);
+  });
+  return rc;
+}
+
+extern "C" int64_t zp_redundancy_raw_workspace(int32_t L, int32_t B, int32_t NB, int32_t BS,
+                                               int32_t Hkv) {
+  return (int64_t)L * B * Hkv * NB * BS * 12;
+}
+
+extern "C" int zp_redundancy_raw(const void* k_cache, const int32_t* block_table, void* red_out,
+                                 void* logits_out, int32_t L, int32_t B, int32_t NB, int32_t BS,
+                                 int32_t Hkv, int32_t D, int32_t num_pages, int64_t k_sl,
+                                 int64_t k_sp, float threshold, double temperature, int32_t dtype,
+                                 void* workspace, int64_t workspace_bytes, void* stream) {
+  int rc = check_common("redundancy_raw", k_cache, block_table, red_out, L, B, NB, BS, Hkv, D,
+                        dtype, k_sl, k_sp);
+  if (rc != ZP_OK) return rc;
+  if (L == 0 || B == 0) return ZP_OK;
+  const int64_t n = (int64_t)L * B * Hkv * NB * BS;
+  ZP_REQUIRE(workspace && workspace_bytes >= n * 12,
+             "redundancy_raw: workspace of %lld bytes required", (long long)n * 12);
+  ZP_REQUIRE(((uintptr_t)workspace % 4) == 0, "redundancy_raw: workspace must be 4-byte aligned");
+  GramArgs a;
+  a.k = (const char*)k_cache; a.table = block_table; a.r_out = nullptr;
+  a.ws_sum = (float*)workspace; a.ws_col = (int32_t*)workspace + n; a.ws_val = (float*)workspace + 2 * n;
+  a.B = B; a.NB = NB; a.BS = BS; a.Hkv = Hkv; a.D = D; a.num_pages = num_pages;
+  a.k_sl = k_sl; a.k_sp = k_sp; a.threshold = threshold; a.eps = 1e-6f;
+  hipStream_t st = (hipStream_t)stream;
+  ZP_DISPATCH_DTYPE(dtype, {
+    rc = launch_gram<T, true>(a, L, st);
+    if (rc != ZP_OK) return rc;
+    rc = launch_softmax<T, true>(red_out, logits_out, block_table, a.ws_sum, a.ws_col, a.ws_val, L,
+                                 B, NB, BS, Hkv, num_pages, temperature, st);
+  });
+  return rc;
+}

@@ -1,0 +1,453 @@
+// Ragged attention scorer: softmax(window queries x paged keys), max over the GQA group,
+// mean (or max) over the window -- one workgroup per (layer, sequence, kv head), MFMA
+// for the QK^T contraction, K tiles staged through double-buffered LDS.
+//
+// The (Hq, W, T) logits the reference materialises are never written (unless the caller
+// asks for them).  The softmax normaliser spans the whole sequence, so the workgroup makes
+// three passes over the sequence's pages, recomputing QK^T each time:
+//   pass 1  row maximum of the (rounded) logits,
+//   pass 2  row sum of exp(rounded(logit - max)),
+//   pass 3  p = exp(.) / sum, max over the group, sum over the window, store.
+// Passes 2 and 3 re-read K from L2 / Infinity Cache.  Rounding points follow the
+// reference (logits, logit-max, softmax output and the window mean are each rounded to the
+// cache dtype), so bf16/fp16 results agree with it to the last bit except where fp32
+// accumulation order moves a value across a rounding boundary.
+//
+// MFMA tiling (wave64, 32x32 tiles): the A operand is a block of 32 query rows, row
+// m = w*Gp + g (Gp = GQA group padded to a power of two), held in registers for the
+// whole pass; the B operand is 32 tokens of the K tile read from LDS.  In the 32x32
+// accumulator layout a lane owns one token column and 16 rows
+// ((r/4)*8 + (lane/32)*4 + r%4), so with this row order the group maximum is taken inside
+// a lane (plus one cross-half exchange when Gp >= 8) and the window sum is a lane-local
+// sum plus one cross-half and one cross-wave (LDS) step.  Wave v of the workgroup owns
+// row block v; tiles of 128 (16-bit) or 64 (fp32) tokens are shared by all waves.
+#include "common.h"
+#include <math.h>
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = 4;
+constexpr int kDmax = 128;
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+template <typename T> struct Mma;
+template <> struct Mma<BF16> {
+  typedef bf16x8_t Frag;
+  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = 128, ROWB = kDmax * 2 + 16;
+  __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mma<F16> {
+  typedef f16x8_t Frag;
+  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = 128, ROWB = kDmax * 2 + 16;
+  __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mma<F32> {
+  typedef float Frag;
+  static constexpr int KPI = 2, EPL = 1, KS = kDmax / KPI, TN = 64, ROWB = kDmax * 4 + 8;
+  __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+  }
+};
+
+struct ScoreArgs {
+  const char* k;
+  const char* q;
+  const int32_t* seq_idx;
+  const int32_t* table;
+  void* out;
+  void* logits;   // optional (L,B,Hq,W,NB,BS)
+  float* ws;      // fp32 (L*B*Hkv, NB*BS) partial window sums, only when row rounds > 1
+  int L, B, NB, BS, Hkv, Hq, G, Gp, D, W, num_pages, max_seqs;
+  int64_t k_sl, k_sp, q_sl, q_ss;  // element strides
+  float scale;
+  int reduce_max;
+  int RB;  // row blocks of 32
+  int gs;  // log2(Gp)
+};
+
+template <typename T>
+__device__ __forceinline__ void zero_frag(typename Mma<T>::Frag& f) {
+  __builtin_memset(&f, 0, sizeof(f));
+}
+
+// exp of a non-positive argument, natural base, via the hardware base-2 exponential.
+__device__ __forceinline__ float exp_neg(float x) {
+  return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void score_kernel(ScoreArgs p) {
+  typedef Mma<T> M;
+  typedef typename M::Frag Frag;
+  constexpr int TN = M::TN, NSUB = TN / 32, ROWB = M::ROWB, KS = M::KS;
+  constexpr int PIECES = kDmax * T::bytes / 16;       // 16-byte pieces per full key row
+  constexpr int ROWS_PER_IT = kThreads / PIECES;      // rows staged per iteration
+  constexpr int STAGE_IT = TN / ROWS_PER_IT;          // iterations (== 8)
+
+  extern __shared__ __align__(16) char smem[];
+  char* kbuf0 = smem;
+  char* kbuf1 = smem + TN * ROWB;
+  float* part = (float*)(smem + 2 * TN * ROWB);        // [kWaves][TN]
+  int* vpage = (int*)(part + kWaves * TN);             // [NB] page id of valid pages
+  int* vslot = vpage + p.NB;                           // [NB] their index in the table (bit 30: last)
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const int h = blockIdx.x % p.Hkv;
+  const int b = (blockIdx.x / p.Hkv) % p.B;
+  const int l = blockIdx.x / (p.Hkv * p.B);
+  const int Tn = p.NB * p.BS;
+  const int64_t orow = (((int64_t)l * p.B + b) * p.Hkv + h);
+
+  // ---- valid page list (block-uniform), zero pad-page outputs
+  __shared__ int nvalid_s;
+  if (tid == 0) {
+    int n = 0;
+    for (int j = 0; j < p.NB; ++j) {
+      const int code = p.table[(int64_t)b * p.NB + j];
+      const int pid = page_is_pad(code) ? -1 : page_id(code);
+      if (pid >= 0 && pid < p.num_pages) {
+        vpage[n] = pid;
+        vslot[n] = j | (page_is_last(code) ? (1 << 30) : 0);
+        ++n;
+      }
+    }
+    nvalid_s = n;
+  }
+  // LDS tiles start zeroed so that head_dim < 128 contributes nothing
+  for (int i = tid; i < 2 * TN * ROWB / 4; i += kThreads) ((uint32_t*)smem)[i] = 0u;
+  __syncthreads();
+  const int nvalid = nvalid_s;
+  {
+    // pad pages (and unusable ids) score exactly 0; their logits stay -inf
+    for (int j = 0; j < p.NB; ++j) {
+      const int code = p.table[(int64_t)b * p.NB + j];
+      const int pid = page_is_pad(code) ? -1 : page_id(code);
+      if (pid >= 0 && pid < p.num_pages) continue;
+      for (int s = tid; s < p.BS; s += kThreads)
+        Elem<T>::st(p.out, orow * Tn + (int64_t)j * p.BS + s, 0.f);
+    }
+  }
+  int seq = p.seq_idx[b];
+  const bool seq_ok = seq >= 0 && seq < p.max_seqs;
+  if (!seq_ok) seq = 0;
+
+  const int tiles_per_page = p.BS / TN;
+  const int ntiles = nvalid * tiles_per_page;
+  const int dpieces = p.D * T::bytes / 16;  // valid 16-byte pieces per key row
+  const int64_t k_row = (int64_t)p.Hkv * p.D * T::bytes;
+  const char* kbase = p.k + (l * p.k_sl) * T::bytes + (int64_t)h * p.D * T::bytes;
+
+  // staging coordinates of this thread
+  const int st_piece = tid % PIECES, st_row0 = tid / PIECES;
+  vec16 pre[STAGE_IT];
+
+  auto issue_loads = [&](int tile) {
+    const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
+    const char* src = kbase + (int64_t)vpage[vp] * p.k_sp * T::bytes + (int64_t)toff * k_row;
+#pragma unroll
+    for (int i = 0; i < STAGE_IT; ++i) {
+      const int row = st_row0 + i * ROWS_PER_IT;
+      if (st_piece < dpieces)
+        pre[i] = *(const vec16*)(src + (int64_t)row * k_row + st_piece * 16);
+    }
+  };
+  auto commit_loads = [&](char* buf) {
+#pragma unroll
+    for (int i = 0; i < STAGE_IT; ++i) {
+      const int row = st_row0 + i * ROWS_PER_IT;
+      if (st_piece < dpieces) {
+        uint2* d = (uint2*)(buf + row * ROWB + st_piece * 16);
+        d[0] = make_uint2(pre[i].x, pre[i].y);
+        d[1] = make_uint2(pre[i].z, pre[i].w);
+      }
+    }
+  };
+
+  const int NR = (p.RB + kWaves - 1) / kWaves;  // row rounds
+  for (int rr = 0; rr < NR; ++rr) {
+    const int rb = rr * kWaves + wave;
+    const bool active = rb < p.RB;
+    // ---- A fragments: query rows of this wave's row block
+    Frag afrag[KS];
+    const int mrow = rb * 32 + col;                 // row this lane loads
+    const int a_w = mrow >> p.gs, a_g = mrow & (p.Gp - 1);
+    const bool a_ok = active && seq_ok && a_w < p.W && a_g < p.G;
+    {
+      const char* qrow = p.q + ((int64_t)l * p.q_sl + (int64_t)seq * p.q_ss +
+                                ((int64_t)a_w * p.Hq + (int64_t)h * p.G + a_g) * p.D) * T::bytes;
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        const int k0 = s * M::KPI + half * M::EPL;
+        if (a_ok && k0 < p.D) afrag[s] = *(const Frag*)(qrow + (int64_t)k0 * T::bytes);
+        else zero_frag<T>(afrag[s]);
+      }
+    }
+    // rows owned by this lane in the accumulator layout
+    float invl[16], mx[16];
+    bool rvalid[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int m = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+      rvalid[r] = active && (m >> p.gs) < p.W && (m & (p.Gp - 1)) < p.G;
+      mx[r] = 0.f;
+      invl[r] = 0.f;
+    }
+
+    for (int pass = 0; pass < 3; ++pass) {
+      float run[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) run[r] = pass == 0 ? -INFINITY : 0.f;
+
+      if (ntiles > 0) {
+        issue_loads(0);
+        commit_loads(kbuf0);
+      }
+      __syncthreads();
+      for (int tile = 0; tile < ntiles; ++tile) {
+        char* cur = (tile & 1) ? kbuf1 : kbuf0;
+        char* nxt = (tile & 1) ? kbuf0 : kbuf1;
+        if (tile + 1 < ntiles) issue_loads(tile + 1);
+
+        const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
+        const int j = vslot[vp] & 0xffff;
+        const bool last = (vslot[vp] >> 30) & 1;
+        float wacc[NSUB];
+        if (active) {
+#pragma unroll
+          for (int st = 0; st < NSUB; ++st) {
+            f32x16_t acc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+            const char* brow = cur + (st * 32 + col) * ROWB + half * M::EPL * T::bytes;
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+              const Frag bf = *(const Frag*)(brow + s * M::KPI * T::bytes);
+              acc = M::mma(afrag[s], bf, acc);
+            }
+            const int slot = toff + st * 32 + col;  // token slot inside its page
+            const bool need_mask = last && (toff + st * 32 + 31 > p.BS - p.W);
+            float pv[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              float sc = acc[r] * p.scale;
+              if (need_mask) {
+                const int m = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+                const int w = m >> p.gs;
+                if (slot > p.BS - p.W + w) sc = -INFINITY;
+              }
+              if (pass == 0) {
+                run[r] = fmaxf(run[r], sc);
+                if (p.logits) pv[r] = Elem<T>::rnd(sc);
+              } else {
+                const float x = Elem<T>::rnd(Elem<T>::rnd(sc) - mx[r]);
+                const float e = exp_neg(x);
+                if (pass == 1) run[r] += e;
+                else pv[r] = Elem<T>::rnd(e * invl[r]);
+              }
+            }
+            if (pass == 0 && p.logits) {
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                const int m = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+                const int w = m >> p.gs, g = m & (p.Gp - 1);
+                if (rvalid[r]) {
+                  const int64_t li =
+                      ((((int64_t)l * p.B + b) * p.Hq + (int64_t)h * p.G + g) * p.W + w) * Tn +
+                      (int64_t)j * p.BS + slot;
+                  Elem<T>::st(p.logits, li, pv[r]);
+                }
+              }
+            }
+            if (pass == 2) {
+              // group max inside the lane, then window sum / max
+              float red;
+              const int Gp = p.Gp;
+              if (Gp >= 4) {
+                float q4[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                  q4[q] = fmaxf(fmaxf(pv[4 * q], pv[4 * q + 1]), fmaxf(pv[4 * q + 2], pv[4 * q + 3]));
+                if (Gp >= 8) {
+#pragma unroll
+                  for (int q = 0; q < 4; ++q) q4[q] = fmaxf(q4[q], __shfl_xor(q4[q], 32, 64));
+                }
+                if (Gp >= 16) {
+                  q4[0] = fmaxf(q4[0], q4[1]);
+                  q4[2] = fmaxf(q4[2], q4[3]);
+                  if (Gp >= 32) red = fmaxf(q4[0], q4[2]);
+                  else red = p.reduce_max ? fmaxf(q4[0], q4[2]) : q4[0] + q4[2];
+                } else {
+                  red = p.reduce_max ? fmaxf(fmaxf(q4[0], q4[1]), fmaxf(q4[2], q4[3]))
+                                     : (q4[0] + q4[1]) + (q4[2] + q4[3]);
+                }
+              } else {
+                float t8[8];
+                if (Gp == 2) {
+#pragma unroll
+                  for (int q = 0; q < 8; ++q) t8[q] = fmaxf(pv[2 * q], pv[2 * q + 1]);
+                } else {
+#pragma unroll
+                  for (int q = 0; q < 8; ++q)
+                    t8[q] = p.reduce_max ? fmaxf(pv[2 * q], pv[2 * q + 1]) : pv[2 * q] + pv[2 * q + 1];
+                }
+                if (p.reduce_max) {
+                  red = fmaxf(fmaxf(fmaxf(t8[0], t8[1]), fmaxf(t8[2], t8[3])),
+                              fmaxf(fmaxf(t8[4], t8[5]), fmaxf(t8[6], t8[7])));
+                } else {
+                  red = ((t8[0] + t8[1]) + (t8[2] + t8[3])) + ((t8[4] + t8[5]) + (t8[6] + t8[7]));
+                }
+              }
+              if (Gp < 8) {  // the two lane halves hold different windows
+                const float o = __shfl_xor(red, 32, 64);
+                red = p.reduce_max ? fmaxf(red, o) : red + o;
+              }
+              wacc[st] = red;
+            }
+          }
+        }
+        if (pass == 2) {
+#pragma unroll
+          for (int st = 0; st < NSUB; ++st)
+            if (half == 0) part[wave * TN + st * 32 + col] = active ? wacc[st] : 0.f;
+          __syncthreads();
+          if (tid < TN) {
+            float v = part[tid];
+#pragma unroll
+            for (int w2 = 1; w2 < kWaves; ++w2)
+              v = p.reduce_max ? fmaxf(v, part[w2 * TN + tid]) : v + part[w2 * TN + tid];
+            const int64_t oi = orow * Tn + (int64_t)j * p.BS + toff + tid;
+            if (NR > 1) {
+              float* wsp = p.ws + oi;
+              if (rr > 0) v = p.reduce_max ? fmaxf(v, *wsp) : v + *wsp;
+              if (rr + 1 < NR) *wsp = v;
+            }
+            if (rr + 1 == NR)
+              Elem<T>::st(p.out, oi, p.reduce_max ? v : Elem<T>::rnd(v / (float)p.W));
+          }
+        }
+        if (tile + 1 < ntiles) commit_loads(nxt);
+        __syncthreads();
+      }
+
+      // ---- end of pass: combine the per-lane row statistics
+      if (pass < 2) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float v = run[r];
+#pragma unroll
+          for (int o = 16; o > 0; o >>= 1) {
+            const float t = __shfl_xor(v, o, 64);
+            v = pass == 0 ? fmaxf(v, t) : v + t;
+          }
+          run[r] = v;
+        }
+        // the xor butterfly leaves the row result in all 32 lanes that share the row
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          if (pass == 0) mx[r] = Elem<T>::rnd(run[r]);
+          else invl[r] = rvalid[r] ? 1.f / run[r] : 0.f;
+        }
+      }
+    }
+  }
+}
+
+}  // namespace
+
+static int pow2_ceil(int v) {
+  int p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+extern "C" int64_t zp_attention_score_workspace(int32_t L, int32_t B, int32_t NB, int32_t BS,
+                                                int32_t Hkv, int32_t Hq, int32_t W) {
+  if (Hkv <= 0 || Hq <= 0) return 0;
+  const int Gp = pow2_ceil(Hq / Hkv);
+  const int RB = (W * Gp + 31) / 32;
+  if (RB <= kWaves) return 0;
+  return (int64_t)L * B * Hkv * NB * BS * 4;
+}
+
+extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
+                                  const int32_t* seq_idx, const int32_t* block_table,
+                                  void* scores_out, void* logits_out, int32_t L, int32_t B,
+                                  int32_t NB, int32_t BS, int32_t Hkv, int32_t Hq, int32_t D,
+                                  int32_t W, int32_t num_pages, int32_t max_seqs, int64_t k_sl,
+                                  int64_t k_sp, int64_t q_sl, int64_t q_ss, float softmax_scale,
+                                  int32_t reduced, int32_t dtype, void* workspace,
+                                  int64_t workspace_bytes, void* stream) {
+  ZP_REQUIRE(k_cache && query_cache && seq_idx && block_table && scores_out,
+             "attention_score: null pointer");
+  ZP_REQUIRE(L >= 0 && B >= 0 && NB > 0 && BS > 0 && Hkv > 0 && Hq > 0 && D > 0 && W > 0,
+             "attention_score: bad dims");
+  ZP_REQUIRE(Hq % Hkv == 0, "attention_score: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
+  ZP_REQUIRE(dtype >= ZP_BF16 && dtype <= ZP_F32, "attention_score: unknown dtype tag %d", dtype);
+  ZP_REQUIRE(reduced == ZP_REDUCE_MEAN || reduced == ZP_REDUCE_MAX,
+             "attention_score: unknown reduction %d", reduced);
+  ZP_REQUIRE(W <= BS, "attention_score: window %d longer than a page of %d", W, BS);
+  const int es = zp_dtype_bytes(dtype);
+  const int TN = dtype == ZP_F32 ? 64 : 128;
+  if (!(D <= kDmax && (D * es) % 16 == 0)) {
+    zp_set_error("attention_score: head_dim %d unsupported (need <= %d and a multiple of %d)", D,
+                 kDmax, 16 / es);
+    return ZP_EUNSUPPORTED;
+  }
+  if (BS % TN != 0) {
+    zp_set_error("attention_score: page size %d is not a multiple of %d", BS, TN);
+    return ZP_EUNSUPPORTED;
+  }
+  const int G = Hq / Hkv, Gp = pow2_ceil(G);
+  if (Gp > 32) {
+    zp_set_error("attention_score: GQA group %d unsupported (max 32)", G);
+    return ZP_EUNSUPPORTED;
+  }
+  ZP_REQUIRE(((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)query_cache % 16) == 0 &&
+                 (k_sl * es) % 16 == 0 && (k_sp * es) % 16 == 0 && (q_sl * es) % 16 == 0 &&
+                 (q_ss * es) % 16 == 0,
+             "attention_score: caches must be 16-byte aligned");
+  ZP_REQUIRE(NB <= 0xffff, "attention_score: too many pages per sequence");
+  if (L == 0 || B == 0) return ZP_OK;
+  const int RB = (W * Gp + 31) / 32;
+  const int64_t need = zp_attention_score_workspace(L, B, NB, BS, Hkv, Hq, W);
+  ZP_REQUIRE(need == 0 || (workspace && workspace_bytes >= need),
+             "attention_score: workspace of %lld bytes required", (long long)need);
+
+  ScoreArgs a;
+  a.k = (const char*)k_cache; a.q = (const char*)query_cache; a.seq_idx = seq_idx;
+  a.table = block_table; a.out = scores_out; a.logits = logits_out; a.ws = (float*)workspace;
+  a.L = L; a.B = B; a.NB = NB; a.BS = BS; a.Hkv = Hkv; a.Hq = Hq; a.G = G; a.Gp = Gp; a.D = D;
+  a.W = W; a.num_pages = num_pages; a.max_seqs = max_seqs;
+  a.k_sl = k_sl; a.k_sp = k_sp; a.q_sl = q_sl; a.q_ss = q_ss;
+  a.scale = softmax_scale; a.reduce_max = reduced == ZP_REDUCE_MAX; a.RB = RB;
+  a.gs = 0;
+  while ((1 << a.gs) < Gp) ++a.gs;
+
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)((int64_t)L * B * Hkv));
+#define ZP_SCORE_LAUNCH()                                                                        \
+  do {                                                                                           \
+    const size_t smem = 2 * (size_t)Mma<T>::TN * Mma<T>::ROWB +                                  \
+                        sizeof(float) * (kWaves * Mma<T>::TN) + sizeof(int) * 2 * NB;            \
+    if (smem > 64 * 1024 &&                                                                      \
+        hipFuncSetAttribute((const void*)score_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                            (int)smem) != hipSuccess) {                                          \
+      zp_set_error("attention_score: cannot reserve %zu bytes of LDS", smem);                    \
+      return ZP_EHIP;                                                                            \
+    }                                                                                            \
+    hipLaunchKernelGGL((score_kernel<T>), grid, dim3(kThreads), smem, st, a);                    \
+  } while (0)
+  ZP_DISPATCH_DTYPE(dtype, ZP_SCORE_LAUNCH());
+#undef ZP_SCORE_LAUNCH
+  ZP_LAUNCH_CHECK();
+  return ZP_OK;
+}
