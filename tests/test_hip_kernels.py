@@ -16,16 +16,20 @@ pytestmark = pytest.mark.gpu
 DTYPES = [torch.float32, torch.bfloat16, torch.float16]
 
 
-def _ulp_close(got, want, dtype, ulps=1, frac_exact=0.0):
-    """got/want: tensors in `dtype`.  Every element within `ulps` units in the last place."""
+def _ulp_close(got, want, dtype, ulps=1, frac_exact=0.0, abs_floor=1e-30):
+    """got/want: tensors in `dtype`.  Every element within `ulps` units in the last place
+    (or within `abs_floor`, for values that are the small remainder of a cancelling sum)."""
     g, w = got.float().cpu(), want.float().cpu()
     assert torch.equal(torch.isinf(g), torch.isinf(w))
     fin = torch.isfinite(w)
     g, w = g[fin], w[fin]
     eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -24}[dtype]
-    tol = ulps * 2 * eps * torch.maximum(w.abs(), g.abs()) + 1e-30
+    tol = ulps * 2 * eps * torch.maximum(w.abs(), g.abs()) + abs_floor
     bad = (g - w).abs() > tol
-    assert not bad.any(), f"{int(bad.sum())} of {bad.numel()} beyond {ulps} ulp; max diff {(g - w).abs().max()}"
+    if bad.any():
+        i = int(((g - w).abs() / tol).argmax())
+        raise AssertionError(f"{int(bad.sum())} of {bad.numel()} beyond {ulps} ulp; worst got {g[i].item()!r} "
+                             f"want {w[i].item()!r}")
     if frac_exact:
         same = (g == w).float().mean().item()
         assert same >= frac_exact, f"only {same:.4f} bit-identical"
@@ -252,8 +256,11 @@ def test_attention_score(dev, dtype, cfg, reduced):
         _rel_close(glog, wlog, rel=1e-4, abs_floor=1e-5)
         _rel_close(got, want, rel=1e-3, abs_floor=1e-9)
     else:
-        _ulp_close(glog, wlog, dtype, ulps=1, frac_exact=0.995)
-        _ulp_close(got, want, dtype, ulps=2, frac_exact=0.9)
+        # near-zero logits are the remainder of a cancelling 128-term sum: fp32 order noise
+        _ulp_close(glog, wlog, dtype, ulps=1, frac_exact=0.995, abs_floor=2e-6)
+        # one logit that rounds the other way moves its probability by exp(ulp(logit)), a
+        # few output ulps; the window mean dilutes that, the window max does not
+        _ulp_close(got, want, dtype, ulps=2 if reduced == "mean" else 16, frac_exact=0.9)
     # without logits the scores are the same bits
     got2 = attention_score(*(a.to(dev) for a in args), reduced=reduced)
     assert torch.equal(got2, got)
@@ -291,7 +298,9 @@ def test_lightning_redundancy(dev, dtype, thr):
         _rel_close(gl, wl, rel=1e-4, abs_floor=1e-3)
         _rel_close(gr, wr, rel=1e-3, abs_floor=1e-9)
     else:
-        _ulp_close(gl, wl, dtype, ulps=1, frac_exact=0.97)
+        # a fully claimed row sums to exactly 0 in the oracle and to fp32 noise of a
+        # ~200-large cancelling sum here: absolute floor
+        _ulp_close(gl, wl, dtype, ulps=1, frac_exact=0.97, abs_floor=1e-3)
         _ulp_close(gr, wr, dtype, ulps=2, frac_exact=0.9)
 
 
@@ -310,5 +319,5 @@ def test_raw_redundancy(dev, dtype):
         _rel_close(gl, wl, rel=1e-4, abs_floor=1e-2)
         _rel_close(gr, wr, rel=1e-3, abs_floor=1e-9)
     else:
-        _ulp_close(gl, wl, dtype, ulps=1)
+        _ulp_close(gl, wl, dtype, ulps=1, abs_floor=1e-2)
         _ulp_close(gr, wr, dtype, ulps=4)

@@ -18,6 +18,8 @@ LIB = os.path.join(HERE, "libzipage_hip.so")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # keep a*b+c as two roundings: the stages restate torch ops that round after each op
+    "-ffp-contract=off",
     "-Wno-unused-command-line-argument",
 ]
 

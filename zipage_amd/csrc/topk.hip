@@ -14,12 +14,14 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
 
-// `low_bit`: keys of this dtype have all bits below it clear (the NaN key keeps that).
+// `low_bit`: the float image of this dtype has all bits below it clear; the key keeps them
+// clear too (for negatives the complement would set them), so the bit search can stop there.
 __device__ __forceinline__ uint32_t score_key(float f, int low_bit) {
   uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0xffffffffu << low_bit;  // NaN sorts largest
-  if (u == 0x80000000u) u = 0u;                             // -0 == +0
-  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+  const uint32_t keep = 0xffffffffu << low_bit;
+  if ((u & 0x7fffffffu) > 0x7f800000u) return keep;  // NaN sorts largest
+  if (u == 0x80000000u) u = 0u;                      // -0 == +0
+  return ((u & 0x80000000u) ? ~u : (u | 0x80000000u)) & keep;
 }
 
 __device__ __forceinline__ int block_count(int c, int* slots /* kWaves */) {
