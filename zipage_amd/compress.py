@@ -1,0 +1,147 @@
+"""One layer chunk of the compression pipeline on the GPU, in the reference's stage order.
+
+Host-side mirror of the body of ``ModelRunner.compress``
+(zipage/engine/model_runner.py:466-622): the same stages with the same switches, each
+dispatched to its HIP entry point.  Nothing here synchronises with the host: the
+reference's ``torch.all(compressed)`` test before pooling (model_runner.py:501) only skips
+work whose result equals its input, so pooling is decided per sequence on the device.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from zipage_amd.kernel.attention_score import attention_score
+from zipage_amd.kernel.compress_kv import compress_kv
+from zipage_amd.kernel.compress_score import compress_score
+from zipage_amd.kernel.global_score import global_score
+from zipage_amd.kernel.lightning_redudancy_score import lightning_redudancy_score
+from zipage_amd.kernel.pooling import pool_scores
+from zipage_amd.kernel.raw_redudancy_score import raw_redudancy_score
+from zipage_amd.kernel.utils import topk_mask
+from zipage_amd.kernel.window_mask import score_epilogue
+
+# stage names as the reference records them (model_runner.py:424-429,624-630)
+STAGES = ("attention_score", "global_score", "pooling", "redudancy_score", "attention_sink",
+          "window_mask", "topk_mask", "compress_kv", "compress_global_score")
+
+
+@dataclass
+class CompressConfig:
+    """The switches of zipage/config.py:22-46 that the compression path reads."""
+    budget_blocks: int = 8            # max_cache_blocks_per_seq
+    query_cache_len: int = 16
+    softmax_scale: float | None = None
+    reduced: str = "mean"
+    use_global_score: bool = False
+    decay_factor: float = 0.8
+    activate_method: str = "max"
+    max_norm: bool = False
+    use_redudancy: bool = False
+    lightning_redudancy: bool = False
+    redudancy_lambda: float = 0.2
+    redudancy_temperature: float = 0.4
+    redudancy_threshold: float = 0.5
+    enable_pooling: bool = False
+    continues_pooling: bool = False
+    pooling_size: int = 5             # the reference runner hard-codes 5 (model_runner.py:71)
+    pooling_mode: str = "max"
+    use_attention_sink: bool = False
+    sink_len: int = 4
+
+
+class StageTimer:
+    """Optional per-stage device timing with the reference's stage names."""
+
+    def __init__(self, enabled: bool):
+        self.enabled = enabled
+        self.spans = []
+
+    def start(self, name):
+        if not self.enabled:
+            return None
+        st, ed = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        st.record()
+        self.spans.append((name, st, ed))
+        return ed
+
+    @staticmethod
+    def stop(ed):
+        if ed is not None:
+            ed.record()
+
+    def seconds(self):
+        """Per-stage totals; call after the stream has been synchronised."""
+        out = {}
+        for name, st, ed in self.spans:
+            out[name] = out.get(name, 0.0) + st.elapsed_time(ed) / 1000.0
+        return out
+
+
+def compress_layers(k_cache, v_cache, query_cache, score_cache, query_ids, block_tables,
+                    compressed, target_block_tables, cfg: CompressConfig, timer=None,
+                    return_intermediates=False):
+    """Score, select and compact one chunk of layers in place.
+
+    k_cache/v_cache: (L, num_pages, BS, Hkv, D); query_cache: (L, max_seqs, W, Hq, D);
+    score_cache: (L, num_pages, BS, Hkv) or None; query_ids: (B,) int32; block_tables:
+    (B, NB) int32 encoded as in model_runner.py:437-463; compressed: (B,) bool;
+    target_block_tables: (B, budget+1) int32.  Returns the keep flag (L, B, Hkv, NB, BS).
+    """
+    t = timer or StageTimer(False)
+    BS = k_cache.shape[2]
+
+    ev = t.start("attention_score")
+    scores = attention_score(k_cache, query_cache, query_ids, block_tables, cfg.softmax_scale,
+                             cfg.reduced)
+    t.stop(ev)
+
+    if cfg.use_global_score:
+        ev = t.start("global_score")
+        if cfg.max_norm:
+            score_epilogue(scores, block_tables, max_norm_scores=True)
+        scores = global_score(scores, score_cache, block_tables, compressed, cfg.decay_factor,
+                              cfg.activate_method)
+        t.stop(ev)
+
+    if cfg.enable_pooling:
+        ev = t.start("pooling")
+        scores = pool_scores(scores, compressed, cfg.pooling_size, cfg.continues_pooling,
+                             cfg.pooling_mode)
+        t.stop(ev)
+
+    red = None
+    if cfg.use_redudancy:
+        ev = t.start("redudancy_score")
+        fn = lightning_redudancy_score if cfg.lightning_redudancy else raw_redudancy_score
+        red = fn(k_cache, block_tables, threshold=cfg.redudancy_threshold,
+                 temperature=cfg.redudancy_temperature)
+        t.stop(ev)
+
+    # combine + sink + window mask + pad mask: one fused pass (window_mask stage)
+    ev = t.start("window_mask")
+    score_epilogue(scores, block_tables, red,
+                   max_norm_red=cfg.use_redudancy and cfg.use_global_score and cfg.max_norm,
+                   redudancy_lambda=cfg.redudancy_lambda,
+                   sink_len=cfg.sink_len if cfg.use_attention_sink else 0,
+                   window=cfg.query_cache_len, mask_pad=True)
+    t.stop(ev)
+
+    ev = t.start("topk_mask")
+    L, B, Hkv, NB, _ = scores.shape
+    flag = topk_mask(scores.view(L, B, Hkv, NB * BS), BS * cfg.budget_blocks)
+    flag = flag.view(L, B, Hkv, NB, BS)
+    t.stop(ev)
+
+    ev = t.start("compress_kv")
+    compress_kv(k_cache, v_cache, flag, block_tables, target_block_tables)
+    t.stop(ev)
+
+    if cfg.use_global_score:
+        ev = t.start("compress_global_score")
+        compress_score(score_cache, flag, block_tables, target_block_tables)
+        t.stop(ev)
+    if return_intermediates:
+        return flag, scores
+    return flag

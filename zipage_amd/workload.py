@@ -1,0 +1,134 @@
+"""Synthetic compression workloads at the benchmark shapes, built directly on the device.
+
+Host bookkeeping follows the reference engine: page tables are encoded as in
+zipage/engine/model_runner.py:437-463, target tables follow ``BlockManager.may_compress``
+(zipage/engine/block_manager.py:129-169): an already-compressed sequence compacts in place
+into its own first ``budget+1`` pages; a first compression behind a shared prefix of ``p``
+pages writes into ``min(p, budget)`` fresh pages followed by its own pages.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+QWEN3_8B = dict(Hq=32, Hkv=8, D=128)
+QWEN3_0_6B = dict(Hq=16, Hkv=8, D=128)
+
+
+@dataclass
+class Workload:
+    name: str
+    k: torch.Tensor            # (L, pages, BS, Hkv, D)
+    v: torch.Tensor
+    q: torch.Tensor            # (L, B, W, Hq, D)
+    score_cache: torch.Tensor | None
+    query_ids: torch.Tensor    # (B,) int32
+    block_tables: torch.Tensor  # (B, NB) int32, encoded
+    compressed: torch.Tensor   # (B,) bool
+    targets: torch.Tensor      # (B, budget+1) int32
+    budget: int
+    W: int
+    tables: list
+
+    @property
+    def B(self):
+        return self.block_tables.shape[0]
+
+    @property
+    def L(self):
+        return self.k.shape[0]
+
+
+def encode_tables(tables, device):
+    width = max(len(t) for t in tables)
+    rows = [list(t[:-1]) + [-t[-1] - 2] + [-1] * (width - len(t)) for t in tables]
+    return torch.tensor(rows, dtype=torch.int32, device=device)
+
+
+def ragged_batch(B, *, L=1, pool_pages=20000, budget=8, W=32, BS=256, dtype=torch.bfloat16,
+                 seed=1, lengths=(2049, 2304), shared_prefix_group=0, shared_prefix_pages=2,
+                 with_score_cache=False, compressed=False, shape=QWEN3_8B, device="cuda:0",
+                 name="ragged"):
+    """B sequences with token counts uniform in ``lengths`` (rounded up to whole pages, since
+    compression fires only on a full last page), pages drawn without replacement from a pool
+    of ``pool_pages`` ids.  With ``shared_prefix_group = n`` every group of n sequences shares
+    its first ``shared_prefix_pages`` pages (copy-on-write targets)."""
+    g = torch.Generator().manual_seed(seed)
+    Hq, Hkv, D = shape["Hq"], shape["Hkv"], shape["D"]
+    lens = torch.randint(lengths[0], lengths[1] + 1, (B,), generator=g)
+    nbs = ((lens + BS - 1) // BS).tolist()
+    perm = torch.randperm(pool_pages, generator=g).tolist()
+    pos = 0
+
+    def take(n):
+        nonlocal pos
+        out = perm[pos:pos + n]
+        pos += n
+        assert len(out) == n, "page pool exhausted"
+        return out
+
+    tables, targets = [], []
+    shared = None
+    for b in range(B):
+        if shared_prefix_group and b % shared_prefix_group == 0:
+            shared = take(shared_prefix_pages)
+        if shared_prefix_group:
+            own = take(nbs[b] - shared_prefix_pages)
+            table = shared + own
+            n_new = min(shared_prefix_pages, budget)
+            fresh = take(n_new)
+            target = fresh + table[shared_prefix_pages:shared_prefix_pages + budget + 1 - n_new]
+        else:
+            table = take(nbs[b])
+            target = table[:budget + 1]
+        tables.append(table)
+        targets.append(target)
+    used = sorted({p for t in tables for p in t})
+    dev = torch.device(device)
+    k = torch.empty((L, pool_pages, BS, Hkv, D), dtype=dtype, device=dev)
+    v = torch.empty((L, pool_pages, BS, Hkv, D), dtype=dtype, device=dev)
+    gg = torch.Generator(device=dev).manual_seed(seed)
+    idx = torch.tensor(used, device=dev)
+    for l in range(L):
+        k[l, idx] = torch.randn((len(used), BS, Hkv, D), generator=gg, device=dev,
+                                dtype=torch.float32).to(dtype)
+        v[l, idx] = torch.randn((len(used), BS, Hkv, D), generator=gg, device=dev,
+                                dtype=torch.float32).to(dtype)
+    q = torch.randn((L, B, W, Hq, D), generator=gg, device=dev, dtype=torch.float32).to(dtype)
+    sc = None
+    if with_score_cache:
+        sc = torch.empty((L, pool_pages, BS, Hkv), dtype=dtype, device=dev)
+        for l in range(L):
+            sc[l, idx] = torch.rand((len(used), BS, Hkv), generator=gg, device=dev).to(dtype)
+    return Workload(
+        name=name, k=k, v=v, q=q, score_cache=sc,
+        query_ids=torch.arange(B, dtype=torch.int32, device=dev),
+        block_tables=encode_tables(tables, dev),
+        compressed=torch.full((B,), bool(compressed), dtype=torch.bool, device=dev),
+        targets=torch.tensor(targets, dtype=torch.int32, device=dev),
+        budget=budget, W=W, tables=tables)
+
+
+def algorithmic_bytes(wl: Workload, cfg) -> dict:
+    """HBM bytes each stage has to move for this workload (per launch over all layers):
+    K once + Q + score out for the scorer; score-cache read+write for the global score;
+    K and V survivors read+written for the compaction."""
+    L, _, BS, Hkv, D = wl.k.shape
+    Hq = wl.q.shape[3]
+    es = wl.k.element_size()
+    valid_pages = sum(len(t) for t in wl.tables)
+    keep = cfg.budget_blocks * BS
+    B = wl.B
+    out = {
+        "attention_score": L * (valid_pages * BS * Hkv * D * es + B * wl.W * Hq * D * es
+                                + valid_pages * BS * Hkv * es),
+        "compress_kv": L * B * 2 * 2 * keep * Hkv * D * es,
+    }
+    if cfg.use_global_score:
+        out["global_score"] = L * 2 * valid_pages * BS * Hkv * es
+        out["compress_global_score"] = L * B * 2 * keep * Hkv * es
+    if cfg.use_redudancy:
+        out["redudancy_score"] = L * valid_pages * BS * Hkv * D * es
+    out["pipeline"] = sum(out.values())
+    return out
