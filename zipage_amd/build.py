@@ -30,7 +30,8 @@ def sources():
 
 def build(verbose: bool = True) -> str:
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    cmd = [hipcc, *FLAGS, *sources(), "-o", LIB + ".tmp"]
+    extra = os.environ.get("ZP_EXTRA_HIPCC_FLAGS", "").split()
+    cmd = [hipcc, *FLAGS, *extra, *sources(), "-o", LIB + ".tmp"]
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)

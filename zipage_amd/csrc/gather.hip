@@ -18,6 +18,12 @@
 namespace {
 
 constexpr int kThreads = 256;
+#ifndef ZP_COMPACT_R
+#define ZP_COMPACT_R 8
+#endif
+// native vector types keep the staged pieces in VGPRs
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ int block_exclusive_scan(int v, int* total, int* lds) {
   const int lane = lane_id(), w = wave_id();
@@ -47,12 +53,16 @@ struct CompactArgs {
   const int32_t* table;
   const int32_t* target;
   int B, NB, BS, Hkv, num_pages, target_width;
+  int n_items;         // L*B*Hkv
   int lpv;             // pieces per token vector
+  int lpv_shift;       // log2(lpv) or -1
+  int bs_shift;        // log2(BS) or -1
   int64_t a_sl, a_sp, a_ss, a_sh;  // byte strides: layer, page, slot, head
   int64_t b_sl, b_sp, b_ss, b_sh;
 };
 
-template <typename P, int R, bool HAS_B>
+// POW2: page size and pieces-per-vector are powers of two, so every index split is a shift.
+template <typename P, int R, bool HAS_B, bool POW2>
 __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
   extern __shared__ __align__(16) char smem[];
   __shared__ int scan_lds[kThreads / 64];
@@ -62,9 +72,11 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
   int* tgt = tab + p.NB;
 
   const int tid = threadIdx.x;
-  const int h = blockIdx.x % p.Hkv;
-  const int b = (blockIdx.x / p.Hkv) % p.B;
-  const int l = blockIdx.x / (p.Hkv * p.B);
+  const int item = zp_xcd_item(p.n_items);
+  if (item >= p.n_items) return;
+  const int h = item % p.Hkv;
+  const int b = (item / p.Hkv) % p.B;
+  const int l = item / (p.Hkv * p.B);
 
   for (int i = tid; i < p.NB; i += kThreads) {
     int code = p.table[(int64_t)b * p.NB + i];
@@ -82,11 +94,12 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
   const int s0 = min(tid * chunk, T), s1 = min(s0 + chunk, T);
   const uint8_t* f = p.flag + (((int64_t)l * p.B + b) * p.Hkv + h) * (int64_t)T;
   int cnt = 0;
-  for (int s = s0; s < s1; ++s) cnt += (f[s] != 0 && tab[s / p.BS] >= 0) ? 1 : 0;
+  auto page_of = [&](int s) { return POW2 ? (s >> p.bs_shift) : (s / p.BS); };
+  for (int s = s0; s < s1; ++s) cnt += (f[s] != 0 && tab[page_of(s)] >= 0) ? 1 : 0;
   int total;
   int off = block_exclusive_scan(cnt, &total, scan_lds);
   for (int s = s0; s < s1; ++s)
-    if (f[s] != 0 && tab[s / p.BS] >= 0) list[off++] = (uint16_t)s;
+    if (f[s] != 0 && tab[page_of(s)] >= 0) list[off++] = (uint16_t)s;
   __syncthreads();
   const int cap = p.target_width * p.BS;
   if (total > cap) total = cap;
@@ -100,16 +113,15 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
     P rb[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int u = base + r * kThreads + tid;
-      if (u < units) {
-        const int i = u / p.lpv, piece = u - i * p.lpv;
-        const int s = list[i];
-        const int j = s / p.BS, slot = s - j * p.BS;
-        const int64_t pid = tab[j];
-        ra[r] = *(const P*)(abase + pid * p.a_sp + slot * p.a_ss + piece * (int)sizeof(P));
-        if (HAS_B)
-          rb[r] = *(const P*)(bbase + pid * p.b_sp + slot * p.b_ss + piece * (int)sizeof(P));
-      }
+      // out-of-range units re-load the last valid piece (never stored): no predicated loads
+      const int u = min(base + r * kThreads + tid, units - 1);
+      const int i = POW2 ? (u >> p.lpv_shift) : (u / p.lpv), piece = u - i * p.lpv;
+      const int s = list[i];
+      const int j = page_of(s), slot = s - j * p.BS;
+      const int64_t pid = tab[j];
+      ra[r] = *(const P*)(abase + pid * p.a_sp + slot * p.a_ss + piece * (int)sizeof(P));
+      if (HAS_B)
+        rb[r] = *(const P*)(bbase + pid * p.b_sp + slot * p.b_ss + piece * (int)sizeof(P));
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -117,8 +129,8 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
     for (int r = 0; r < R; ++r) {
       const int u = base + r * kThreads + tid;
       if (u < units) {
-        const int i = u / p.lpv, piece = u - i * p.lpv;
-        const int j = i / p.BS, slot = i - j * p.BS;
+        const int i = POW2 ? (u >> p.lpv_shift) : (u / p.lpv), piece = u - i * p.lpv;
+        const int j = page_of(i), slot = i - j * p.BS;
         const int64_t pid = tgt[j];
         if (pid >= 0) {
           *(P*)(abase + pid * p.a_sp + slot * p.a_ss + piece * (int)sizeof(P)) = ra[r];
@@ -130,22 +142,38 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
   }
 }
 
-template <typename P, int R, bool HAS_B>
-int launch_compact(const CompactArgs& a, int L, hipStream_t st) {
+static int log2_exact(int v) {
+  if (v <= 0 || (v & (v - 1))) return -1;
+  int s = 0;
+  while ((1 << s) < v) ++s;
+  return s;
+}
+
+template <typename P, int R, bool HAS_B, bool POW2>
+int launch_compact_impl(CompactArgs a, int L, hipStream_t st) {
+  a.n_items = L * a.B * a.Hkv;
   const int T = a.NB * a.BS;
   size_t smem = (((size_t)T * 2 + 15) & ~(size_t)15) + sizeof(int) * (a.NB + a.target_width);
-  dim3 grid((unsigned)((int64_t)L * a.B * a.Hkv));
+  dim3 grid(zp_xcd_grid((int64_t)L * a.B * a.Hkv));
   if (smem > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)compact_kernel<P, R, HAS_B>,
+    hipError_t e = hipFuncSetAttribute((const void*)compact_kernel<P, R, HAS_B, POW2>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) {
       zp_set_error("compaction: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
       return ZP_EHIP;
     }
   }
-  hipLaunchKernelGGL((compact_kernel<P, R, HAS_B>), grid, dim3(kThreads), smem, st, a);
+  hipLaunchKernelGGL((compact_kernel<P, R, HAS_B, POW2>), grid, dim3(kThreads), smem, st, a);
   ZP_LAUNCH_CHECK();
   return ZP_OK;
+}
+
+template <typename P, int R, bool HAS_B>
+int launch_compact(CompactArgs a, int L, hipStream_t st) {
+  a.lpv_shift = log2_exact(a.lpv);
+  a.bs_shift = log2_exact(a.BS);
+  if (a.lpv_shift >= 0 && a.bs_shift >= 0) return launch_compact_impl<P, R, HAS_B, true>(a, L, st);
+  return launch_compact_impl<P, R, HAS_B, false>(a, L, st);
 }
 
 inline bool aligned_to(int64_t v, int n) { return (v % n) == 0; }
@@ -205,8 +233,8 @@ extern "C" int zp_compress_kv(void* key, void* value, const uint8_t* flag,
   ZP_REQUIRE((int64_t)target_width * BS * a.lpv < (int64_t)1 << 31, "compress_kv: row too large");
   hipStream_t st = (hipStream_t)stream;
   switch (piece) {
-    case 16: return launch_compact<vec16, 8, true>(a, L, st);
-    case 8:  return launch_compact<uint2, 8, true>(a, L, st);
+    case 16: return launch_compact<u32x4, ZP_COMPACT_R, true>(a, L, st);
+    case 8:  return launch_compact<u32x2, 8, true>(a, L, st);
     case 4:  return launch_compact<uint32_t, 8, true>(a, L, st);
     default: return launch_compact<uint16_t, 8, true>(a, L, st);
   }
@@ -267,8 +295,8 @@ extern "C" int zp_store_query(const void* query, void* query_cache, const int32_
                      (const char*)query, (char*)query_cache, slot_mapping, pieces, num_tokens, \
                      max_seqs, window, qs, cs, cl, sm_stride_row, sm_stride_col)
   switch (piece) {
-    case 16: ZP_SQ(vec16); break;
-    case 8:  ZP_SQ(uint2); break;
+    case 16: ZP_SQ(u32x4); break;
+    case 8:  ZP_SQ(u32x2); break;
     case 4:  ZP_SQ(uint32_t); break;
     default: ZP_SQ(uint16_t); break;
   }
