@@ -23,6 +23,7 @@
 // row block v; tiles of 128 (16-bit) or 64 (fp32) tokens are shared by all waves.
 #include "common.h"
 #include <math.h>
+#include <type_traits>
 
 namespace {
 
@@ -78,13 +79,37 @@ __device__ __forceinline__ void zero_frag(typename Mma<T>::Frag& f) {
   __builtin_memset(&f, 0, sizeof(f));
 }
 
+// Round two fp32 values to the cache dtype and back, in place.  bf16 uses the packed
+// hardware conversion (one instruction for the pair).
+template <typename T> struct Rnd;
+template <> struct Rnd<F32> {
+  __device__ static __forceinline__ void pair(float&, float&) {}
+};
+template <> struct Rnd<BF16> {
+  __device__ static __forceinline__ void pair(float& a, float& b) {
+    typedef __attribute__((ext_vector_type(2))) float f2;
+    typedef __attribute__((ext_vector_type(2))) __bf16 b2;
+    const f2 v = {a, b};
+    const b2 r = __builtin_convertvector(v, b2);
+    const uint32_t u = __builtin_bit_cast(uint32_t, r);
+    a = __uint_as_float(u << 16);
+    b = __uint_as_float(u & 0xffff0000u);
+  }
+};
+template <> struct Rnd<F16> {
+  __device__ static __forceinline__ void pair(float& a, float& b) {
+    a = (float)(_Float16)a;
+    b = (float)(_Float16)b;
+  }
+};
+
 // exp of a non-positive argument, natural base, via the hardware base-2 exponential.
 __device__ __forceinline__ float exp_neg(float x) {
   return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
 }
 
 template <typename T>
-__global__ __launch_bounds__(kThreads) void score_kernel(ScoreArgs p) {
+__global__ __launch_bounds__(kThreads, (T::bytes == 2 ? 2 : 1)) void score_kernel(ScoreArgs p) {
   typedef Mma<T> M;
   typedef typename M::Frag Frag;
   constexpr int TN = M::TN, NSUB = TN / 32, ROWB = M::ROWB, KS = M::KS;
@@ -173,6 +198,8 @@ __global__ __launch_bounds__(kThreads) void score_kernel(ScoreArgs p) {
   };
 
   const int NR = (p.RB + kWaves - 1) / kWaves;  // row rounds
+  const float ascale = fabsf(p.scale);
+  const float sgn = p.scale < 0.f ? -1.f : 1.f;
   for (int rr = 0; rr < NR; ++rr) {
     const int rb = rr * kWaves + wave;
     const bool active = rb < p.RB;
@@ -191,22 +218,18 @@ __global__ __launch_bounds__(kThreads) void score_kernel(ScoreArgs p) {
         else zero_frag<T>(afrag[s]);
       }
     }
-    // rows owned by this lane in the accumulator layout
+    // rows owned by this lane in the accumulator layout: (r/4)*8 + half*4 + r%4
+    const int row0 = rb * 32 + half * 4;
     float invl[16], mx[16];
-    bool rvalid[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int m = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-      rvalid[r] = active && (m >> p.gs) < p.W && (m & (p.Gp - 1)) < p.G;
-      mx[r] = 0.f;
-      invl[r] = 0.f;
-    }
+    for (int r = 0; r < 16; ++r) { mx[r] = 0.f; invl[r] = 0.f; }
 
-    for (int pass = 0; pass < 3; ++pass) {
+    // One sweep over the sequence's K tiles.  PASS 0: row max; 1: row sum of exp; 2: output.
+    auto sweep = [&](auto pass_c) {
+      constexpr int PASS = decltype(pass_c)::value;
       float run[16];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) run[r] = pass == 0 ? -INFINITY : 0.f;
-
+      for (int r = 0; r < 16; ++r) run[r] = PASS == 0 ? -INFINITY : 0.f;
       if (ntiles > 0) {
         issue_loads(0);
         commit_loads(kbuf0);
@@ -216,13 +239,11 @@ __global__ __launch_bounds__(kThreads) void score_kernel(ScoreArgs p) {
         char* cur = (tile & 1) ? kbuf1 : kbuf0;
         char* nxt = (tile & 1) ? kbuf0 : kbuf1;
         if (tile + 1 < ntiles) issue_loads(tile + 1);
-
         const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
         const int j = vslot[vp] & 0xffff;
         const bool last = (vslot[vp] >> 30) & 1;
-        float wacc[NSUB];
         if (active) {
-#pragma unroll
+#pragma unroll 1
           for (int st = 0; st < NSUB; ++st) {
             f32x16_t acc;
 #pragma unroll
@@ -234,90 +255,103 @@ __global__ __launch_bounds__(kThreads) void score_kernel(ScoreArgs p) {
               acc = M::mma(afrag[s], bf, acc);
             }
             const int slot = toff + st * 32 + col;  // token slot inside its page
-            const bool need_mask = last && (toff + st * 32 + 31 > p.BS - p.W);
-            float pv[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              float sc = acc[r] * p.scale;
-              if (need_mask) {
-                const int m = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-                const int w = m >> p.gs;
-                if (slot > p.BS - p.W + w) sc = -INFINITY;
-              }
-              if (pass == 0) {
-                run[r] = fmaxf(run[r], sc);
-                if (p.logits) pv[r] = Elem<T>::rnd(sc);
-              } else {
-                const float x = Elem<T>::rnd(Elem<T>::rnd(sc) - mx[r]);
-                const float e = exp_neg(x);
-                if (pass == 1) run[r] += e;
-                else pv[r] = Elem<T>::rnd(e * invl[r]);
-              }
-            }
-            if (pass == 0 && p.logits) {
+            // causal mask: only the tail of the last page can be hidden from a window row
+            if (last && (toff + st * 32 + 31 > p.BS - p.W)) {
 #pragma unroll
               for (int r = 0; r < 16; ++r) {
-                const int m = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-                const int w = m >> p.gs, g = m & (p.Gp - 1);
-                if (rvalid[r]) {
-                  const int64_t li =
-                      ((((int64_t)l * p.B + b) * p.Hq + (int64_t)h * p.G + g) * p.W + w) * Tn +
-                      (int64_t)j * p.BS + slot;
-                  Elem<T>::st(p.logits, li, pv[r]);
-                }
+                const int w = (row0 + (r >> 2) * 8 + (r & 3)) >> p.gs;
+                if (slot > p.BS - p.W + w) acc[r] = -sgn * INFINITY;
               }
             }
-            if (pass == 2) {
-              // group max inside the lane, then window sum / max
-              float red;
-              const int Gp = p.Gp;
-              if (Gp >= 4) {
-                float q4[4];
+            if constexpr (PASS == 0) {
+              // max of sign(scale)*acc; scaling is monotone, so it is applied once at the end
 #pragma unroll
-                for (int q = 0; q < 4; ++q)
-                  q4[q] = fmaxf(fmaxf(pv[4 * q], pv[4 * q + 1]), fmaxf(pv[4 * q + 2], pv[4 * q + 3]));
-                if (Gp >= 8) {
+              for (int r = 0; r < 16; ++r) run[r] = fmaxf(run[r], sgn * acc[r]);
+              if (p.logits) {
 #pragma unroll
-                  for (int q = 0; q < 4; ++q) q4[q] = fmaxf(q4[q], __shfl_xor(q4[q], 32, 64));
-                }
-                if (Gp >= 16) {
-                  q4[0] = fmaxf(q4[0], q4[1]);
-                  q4[2] = fmaxf(q4[2], q4[3]);
-                  if (Gp >= 32) red = fmaxf(q4[0], q4[2]);
-                  else red = p.reduce_max ? fmaxf(q4[0], q4[2]) : q4[0] + q4[2];
-                } else {
-                  red = p.reduce_max ? fmaxf(fmaxf(q4[0], q4[1]), fmaxf(q4[2], q4[3]))
-                                     : (q4[0] + q4[1]) + (q4[2] + q4[3]);
-                }
-              } else {
-                float t8[8];
-                if (Gp == 2) {
-#pragma unroll
-                  for (int q = 0; q < 8; ++q) t8[q] = fmaxf(pv[2 * q], pv[2 * q + 1]);
-                } else {
-#pragma unroll
-                  for (int q = 0; q < 8; ++q)
-                    t8[q] = p.reduce_max ? fmaxf(pv[2 * q], pv[2 * q + 1]) : pv[2 * q] + pv[2 * q + 1];
-                }
-                if (p.reduce_max) {
-                  red = fmaxf(fmaxf(fmaxf(t8[0], t8[1]), fmaxf(t8[2], t8[3])),
-                              fmaxf(fmaxf(t8[4], t8[5]), fmaxf(t8[6], t8[7])));
-                } else {
-                  red = ((t8[0] + t8[1]) + (t8[2] + t8[3])) + ((t8[4] + t8[5]) + (t8[6] + t8[7]));
+                for (int r = 0; r < 16; ++r) {
+                  const int m = row0 + (r >> 2) * 8 + (r & 3);
+                  const int w = m >> p.gs, g = m & (p.Gp - 1);
+                  if (w < p.W && g < p.G) {
+                    const int64_t li =
+                        ((((int64_t)l * p.B + b) * p.Hq + (int64_t)h * p.G + g) * p.W + w) * Tn +
+                        (int64_t)j * p.BS + slot;
+                    Elem<T>::st(p.logits, li, acc[r] * p.scale);
+                  }
                 }
               }
-              if (Gp < 8) {  // the two lane halves hold different windows
-                const float o = __shfl_xor(red, 32, 64);
-                red = p.reduce_max ? fmaxf(red, o) : red + o;
+            } else {
+              float pv[16];
+#pragma unroll
+              for (int r = 0; r < 16; r += 2) {
+                float s0 = acc[r] * p.scale, s1 = acc[r + 1] * p.scale;
+                Rnd<T>::pair(s0, s1);
+                float x0 = s0 - mx[r], x1 = s1 - mx[r + 1];
+                Rnd<T>::pair(x0, x1);
+                const float e0 = exp_neg(x0), e1 = exp_neg(x1);
+                if constexpr (PASS == 1) {
+                  run[r] += e0;
+                  run[r + 1] += e1;
+                } else {
+                  float p0 = e0 * invl[r], p1 = e1 * invl[r + 1];
+                  Rnd<T>::pair(p0, p1);
+                  pv[r] = p0;
+                  pv[r + 1] = p1;
+                }
               }
-              wacc[st] = red;
+              if constexpr (PASS == 2) {
+                // group max inside the lane, then window sum / max
+                float red;
+                const int Gp = p.Gp;
+                if (Gp >= 4) {
+                  float q4[4];
+#pragma unroll
+                  for (int q = 0; q < 4; ++q)
+                    q4[q] = fmaxf(fmaxf(pv[4 * q], pv[4 * q + 1]), fmaxf(pv[4 * q + 2], pv[4 * q + 3]));
+                  if (Gp >= 8) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) q4[q] = fmaxf(q4[q], __shfl_xor(q4[q], 32, 64));
+                  }
+                  if (Gp >= 16) {
+                    q4[0] = fmaxf(q4[0], q4[1]);
+                    q4[2] = fmaxf(q4[2], q4[3]);
+                    if (Gp >= 32) red = fmaxf(q4[0], q4[2]);
+                    else red = p.reduce_max ? fmaxf(q4[0], q4[2]) : q4[0] + q4[2];
+                  } else {
+                    red = p.reduce_max ? fmaxf(fmaxf(q4[0], q4[1]), fmaxf(q4[2], q4[3]))
+                                       : (q4[0] + q4[1]) + (q4[2] + q4[3]);
+                  }
+                } else {
+                  float t8[8];
+                  if (Gp == 2) {
+#pragma unroll
+                    for (int q = 0; q < 8; ++q) t8[q] = fmaxf(pv[2 * q], pv[2 * q + 1]);
+                  } else {
+#pragma unroll
+                    for (int q = 0; q < 8; ++q)
+                      t8[q] = p.reduce_max ? fmaxf(pv[2 * q], pv[2 * q + 1]) : pv[2 * q] + pv[2 * q + 1];
+                  }
+                  if (p.reduce_max) {
+                    red = fmaxf(fmaxf(fmaxf(t8[0], t8[1]), fmaxf(t8[2], t8[3])),
+                                fmaxf(fmaxf(t8[4], t8[5]), fmaxf(t8[6], t8[7])));
+                  } else {
+                    red = ((t8[0] + t8[1]) + (t8[2] + t8[3])) + ((t8[4] + t8[5]) + (t8[6] + t8[7]));
+                  }
+                }
+                if (Gp < 8) {  // the two lane halves hold different windows
+                  const float o = __shfl_xor(red, 32, 64);
+                  red = p.reduce_max ? fmaxf(red, o) : red + o;
+                }
+                if (half == 0) part[wave * TN + st * 32 + col] = red;
+              }
             }
           }
-        }
-        if (pass == 2) {
+        } else if (PASS == 2) {
 #pragma unroll
           for (int st = 0; st < NSUB; ++st)
-            if (half == 0) part[wave * TN + st * 32 + col] = active ? wacc[st] : 0.f;
+            if (half == 0) part[wave * TN + st * 32 + col] = 0.f;
+        }
+        if constexpr (PASS == 2) {
           __syncthreads();
           if (tid < TN) {
             float v = part[tid];
@@ -337,27 +371,29 @@ __global__ __launch_bounds__(kThreads) void score_kernel(ScoreArgs p) {
         if (tile + 1 < ntiles) commit_loads(nxt);
         __syncthreads();
       }
-
-      // ---- end of pass: combine the per-lane row statistics
-      if (pass < 2) {
+      // the xor butterfly leaves the row result in all 32 lanes that share the row
+      if constexpr (PASS < 2) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           float v = run[r];
 #pragma unroll
           for (int o = 16; o > 0; o >>= 1) {
             const float t = __shfl_xor(v, o, 64);
-            v = pass == 0 ? fmaxf(v, t) : v + t;
+            v = PASS == 0 ? fmaxf(v, t) : v + t;
           }
-          run[r] = v;
-        }
-        // the xor butterfly leaves the row result in all 32 lanes that share the row
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          if (pass == 0) mx[r] = Elem<T>::rnd(run[r]);
-          else invl[r] = rvalid[r] ? 1.f / run[r] : 0.f;
+          if constexpr (PASS == 0) {
+            mx[r] = Elem<T>::rnd(v * ascale);
+          } else {
+            const int m = row0 + (r >> 2) * 8 + (r & 3);
+            const bool ok = active && (m >> p.gs) < p.W && (m & (p.Gp - 1)) < p.G;
+            invl[r] = ok ? 1.f / v : 0.f;
+          }
         }
       }
-    }
+    };
+    sweep(std::integral_constant<int, 0>{});
+    sweep(std::integral_constant<int, 1>{});
+    sweep(std::integral_constant<int, 2>{});
   }
 }
 
