@@ -27,8 +27,10 @@
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kWaves = 4;
+constexpr int kThreads = 512;
+constexpr int kWaves = 8;      // waves per workgroup
+constexpr int kRowWaves = 4;   // waves along the query-row axis; the other factor splits tokens
+constexpr int kTokWaves = kWaves / kRowWaves;
 constexpr int kDmax = 128;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -38,21 +40,21 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 template <typename T> struct Mma;
 template <> struct Mma<BF16> {
   typedef bf16x8_t Frag;
-  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = 128, ROWB = kDmax * 2 + 16;
+  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = 256, ROWB = kDmax * 2 + 16;
   __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
 };
 template <> struct Mma<F16> {
   typedef f16x8_t Frag;
-  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = 128, ROWB = kDmax * 2 + 16;
+  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = 256, ROWB = kDmax * 2 + 16;
   __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
 };
 template <> struct Mma<F32> {
   typedef float Frag;
-  static constexpr int KPI = 2, EPL = 1, KS = kDmax / KPI, TN = 64, ROWB = kDmax * 4 + 8;
+  static constexpr int KPI = 2, EPL = 1, KS = kDmax / KPI, TN = 128, ROWB = kDmax * 4 + 8;
   __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
   }
@@ -87,6 +89,9 @@ template <> struct Rnd<F32> {
 };
 template <> struct Rnd<BF16> {
   __device__ static __forceinline__ void pair(float& a, float& b) {
+#ifdef ZP_DBG_NORND
+    return;
+#endif
     typedef __attribute__((ext_vector_type(2))) float f2;
     typedef __attribute__((ext_vector_type(2))) __bf16 b2;
     const f2 v = {a, b};
@@ -105,14 +110,17 @@ template <> struct Rnd<F16> {
 
 // exp of a non-positive argument, natural base, via the hardware base-2 exponential.
 __device__ __forceinline__ float exp_neg(float x) {
+#ifdef ZP_DBG_NOEXP
+  return x * 1.44269504088896340736f;
+#endif
   return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
 }
 
-template <typename T>
-__global__ __launch_bounds__(kThreads, (T::bytes == 2 ? 2 : 1)) void score_kernel(ScoreArgs p) {
+template <typename T, bool LOGITS>
+__global__ __launch_bounds__(kThreads) void score_kernel(ScoreArgs p) {
   typedef Mma<T> M;
   typedef typename M::Frag Frag;
-  constexpr int TN = M::TN, NSUB = TN / 32, ROWB = M::ROWB, KS = M::KS;
+  constexpr int TN = M::TN, NSUB = TN / 32 / kTokWaves, ROWB = M::ROWB, KS = M::KS;
   constexpr int PIECES = kDmax * T::bytes / 16;       // 16-byte pieces per full key row
   constexpr int ROWS_PER_IT = kThreads / PIECES;      // rows staged per iteration
   constexpr int STAGE_IT = TN / ROWS_PER_IT;          // iterations (== 8)
@@ -120,12 +128,14 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? 2 : 1)) void score_kerne
   extern __shared__ __align__(16) char smem[];
   char* kbuf0 = smem;
   char* kbuf1 = smem + TN * ROWB;
-  float* part = (float*)(smem + 2 * TN * ROWB);        // [kWaves][TN]
-  int* vpage = (int*)(part + kWaves * TN);             // [NB] page id of valid pages
+  float* part = (float*)(smem + 2 * TN * ROWB);        // [2][kRowWaves][TN]
+  float* stat = part + 2 * kRowWaves * TN;              // [kWaves][32] row statistics
+  int* vpage = (int*)(stat + kWaves * 32);             // [NB] page id of valid pages
   int* vslot = vpage + p.NB;                           // [NB] their index in the table (bit 30: last)
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
+  const int rbw = wave % kRowWaves, tg = wave / kRowWaves;  // row-block wave, token group
   const int h = blockIdx.x % p.Hkv;
   const int b = (blockIdx.x / p.Hkv) % p.B;
   const int l = blockIdx.x / (p.Hkv * p.B);
@@ -176,6 +186,9 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? 2 : 1)) void score_kerne
   vec16 pre[STAGE_IT];
 
   auto issue_loads = [&](int tile) {
+#ifdef ZP_DBG_NOLOAD
+    return;
+#endif
     const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
     const char* src = kbase + (int64_t)vpage[vp] * p.k_sp * T::bytes + (int64_t)toff * k_row;
 #pragma unroll
@@ -197,11 +210,11 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? 2 : 1)) void score_kerne
     }
   };
 
-  const int NR = (p.RB + kWaves - 1) / kWaves;  // row rounds
+  const int NR = (p.RB + kRowWaves - 1) / kRowWaves;  // row rounds
   const float ascale = fabsf(p.scale);
   const float sgn = p.scale < 0.f ? -1.f : 1.f;
   for (int rr = 0; rr < NR; ++rr) {
-    const int rb = rr * kWaves + wave;
+    const int rb = rr * kRowWaves + rbw;
     const bool active = rb < p.RB;
     // ---- A fragments: query rows of this wave's row block
     Frag afrag[KS];
@@ -218,6 +231,10 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? 2 : 1)) void score_kerne
         else zero_frag<T>(afrag[s]);
       }
     }
+    // the query fragments are complete before the tile loop starts, so waits inside it only
+    // concern that loop's own loads
+#pragma unroll
+    for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(afrag[s]));
     // rows owned by this lane in the accumulator layout: (r/4)*8 + half*4 + r%4
     const int row0 = rb * 32 + half * 4;
     float invl[16], mx[16];
@@ -227,6 +244,23 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? 2 : 1)) void score_kerne
     // One sweep over the sequence's K tiles.  PASS 0: row max; 1: row sum of exp; 2: output.
     auto sweep = [&](auto pass_c) {
       constexpr int PASS = decltype(pass_c)::value;
+      auto finish_tile = [&](int tile, int j, int toff) {
+        if (tid < TN) {
+          const float* pt = part + (tile & 1) * kRowWaves * TN;
+          float v = pt[tid];
+#pragma unroll
+          for (int w2 = 1; w2 < kRowWaves; ++w2)
+            v = p.reduce_max ? fmaxf(v, pt[w2 * TN + tid]) : v + pt[w2 * TN + tid];
+          const int64_t oi = orow * Tn + (int64_t)j * p.BS + toff + tid;
+          if (NR > 1) {
+            float* wsp = p.ws + oi;
+            if (rr > 0) v = p.reduce_max ? fmaxf(v, *wsp) : v + *wsp;
+            if (rr + 1 < NR) *wsp = v;
+          }
+          if (rr + 1 == NR)
+            Elem<T>::st(p.out, oi, p.reduce_max ? v : Elem<T>::rnd(v / (float)p.W));
+        }
+      };
       float run[16];
 #pragma unroll
       for (int r = 0; r < 16; ++r) run[r] = PASS == 0 ? -INFINITY : 0.f;
@@ -242,17 +276,28 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? 2 : 1)) void score_kerne
         const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
         const int j = vslot[vp] & 0xffff;
         const bool last = (vslot[vp] >> 30) & 1;
+#ifdef ZP_DBG_NOCOMPUTE
+        if (false) {
+#else
         if (active) {
+#endif
 #pragma unroll 1
-          for (int st = 0; st < NSUB; ++st) {
+          for (int sti = 0; sti < NSUB; ++sti) {
+            const int st = tg * NSUB + sti;
             f32x16_t acc;
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[r] = 0.f;
             const char* brow = cur + (st * 32 + col) * ROWB + half * M::EPL * T::bytes;
+            // all B fragments of the subtile are requested before the first MFMA needs one
+            constexpr int KB = KS < 8 ? KS : 8;
 #pragma unroll
-            for (int s = 0; s < KS; ++s) {
-              const Frag bf = *(const Frag*)(brow + s * M::KPI * T::bytes);
-              acc = M::mma(afrag[s], bf, acc);
+            for (int s0 = 0; s0 < KS; s0 += KB) {
+              Frag bfr[KB];
+#pragma unroll
+              for (int s = 0; s < KB; ++s) bfr[s] = *(const Frag*)(brow + (s0 + s) * M::KPI * T::bytes);
+              __builtin_amdgcn_sched_barrier(0);  // keep the reads grouped ahead of the MFMAs
+#pragma unroll
+              for (int s = 0; s < KB; ++s) acc = M::mma(afrag[s0 + s], bfr[s], acc);
             }
             const int slot = toff + st * 32 + col;  // token slot inside its page
             // causal mask: only the tail of the last page can be hidden from a window row
@@ -267,7 +312,7 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? 2 : 1)) void score_kerne
               // max of sign(scale)*acc; scaling is monotone, so it is applied once at the end
 #pragma unroll
               for (int r = 0; r < 16; ++r) run[r] = fmaxf(run[r], sgn * acc[r]);
-              if (p.logits) {
+              if constexpr (LOGITS) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                   const int m = row0 + (r >> 2) * 8 + (r & 3);
@@ -342,36 +387,23 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? 2 : 1)) void score_kerne
                   const float o = __shfl_xor(red, 32, 64);
                   red = p.reduce_max ? fmaxf(red, o) : red + o;
                 }
-                if (half == 0) part[wave * TN + st * 32 + col] = red;
+                if (half == 0) part[((tile & 1) * kRowWaves + rbw) * TN + st * 32 + col] = red;
               }
             }
           }
         } else if (PASS == 2) {
 #pragma unroll
-          for (int st = 0; st < NSUB; ++st)
-            if (half == 0) part[wave * TN + st * 32 + col] = 0.f;
-        }
-        if constexpr (PASS == 2) {
-          __syncthreads();
-          if (tid < TN) {
-            float v = part[tid];
-#pragma unroll
-            for (int w2 = 1; w2 < kWaves; ++w2)
-              v = p.reduce_max ? fmaxf(v, part[w2 * TN + tid]) : v + part[w2 * TN + tid];
-            const int64_t oi = orow * Tn + (int64_t)j * p.BS + toff + tid;
-            if (NR > 1) {
-              float* wsp = p.ws + oi;
-              if (rr > 0) v = p.reduce_max ? fmaxf(v, *wsp) : v + *wsp;
-              if (rr + 1 < NR) *wsp = v;
-            }
-            if (rr + 1 == NR)
-              Elem<T>::st(p.out, oi, p.reduce_max ? v : Elem<T>::rnd(v / (float)p.W));
-          }
+          for (int sti = 0; sti < NSUB; ++sti)
+            if (half == 0) part[((tile & 1) * kRowWaves + rbw) * TN + (tg * NSUB + sti) * 32 + col] = 0.f;
         }
         if (tile + 1 < ntiles) commit_loads(nxt);
         __syncthreads();
+        // the window partials of this tile are complete: combine the waves' shares while the
+        // next tile is being computed (the buffer is rewritten two tiles later)
+        if constexpr (PASS == 2) finish_tile(tile, j, toff);
       }
-      // the xor butterfly leaves the row result in all 32 lanes that share the row
+      // the xor butterfly leaves the row result in all 32 lanes that share the row; the
+      // token-group waves that share a row block then combine their halves through LDS
       if constexpr (PASS < 2) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -379,6 +411,19 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? 2 : 1)) void score_kerne
 #pragma unroll
           for (int o = 16; o > 0; o >>= 1) {
             const float t = __shfl_xor(v, o, 64);
+            v = PASS == 0 ? fmaxf(v, t) : v + t;
+          }
+          run[r] = v;
+          if (col == 0) stat[wave * 32 + (r >> 2) * 8 + half * 4 + (r & 3)] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float v = run[r];
+#pragma unroll
+          for (int g2 = 1; g2 < kTokWaves; ++g2) {
+            const int ow = ((tg + g2) % kTokWaves) * kRowWaves + rbw;
+            const float t = stat[ow * 32 + (r >> 2) * 8 + half * 4 + (r & 3)];
             v = PASS == 0 ? fmaxf(v, t) : v + t;
           }
           if constexpr (PASS == 0) {
@@ -389,11 +434,15 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? 2 : 1)) void score_kerne
             invl[r] = ok ? 1.f / v : 0.f;
           }
         }
+        __syncthreads();
       }
     };
-    sweep(std::integral_constant<int, 0>{});
-    sweep(std::integral_constant<int, 1>{});
-    sweep(std::integral_constant<int, 2>{});
+#ifndef ZP_DBG_SWEEPS
+#define ZP_DBG_SWEEPS 7
+#endif
+    if (ZP_DBG_SWEEPS & 1) sweep(std::integral_constant<int, 0>{});
+    if (ZP_DBG_SWEEPS & 2) sweep(std::integral_constant<int, 1>{});
+    if (ZP_DBG_SWEEPS & 4) sweep(std::integral_constant<int, 2>{});
   }
 }
 
@@ -410,7 +459,7 @@ extern "C" int64_t zp_attention_score_workspace(int32_t L, int32_t B, int32_t NB
   if (Hkv <= 0 || Hq <= 0) return 0;
   const int Gp = pow2_ceil(Hq / Hkv);
   const int RB = (W * Gp + 31) / 32;
-  if (RB <= kWaves) return 0;
+  if (RB <= kRowWaves) return 0;
   return (int64_t)L * B * Hkv * NB * BS * 4;
 }
 
@@ -432,7 +481,7 @@ extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
              "attention_score: unknown reduction %d", reduced);
   ZP_REQUIRE(W <= BS, "attention_score: window %d longer than a page of %d", W, BS);
   const int es = zp_dtype_bytes(dtype);
-  const int TN = dtype == ZP_F32 ? 64 : 128;
+  const int TN = dtype == ZP_F32 ? 128 : 256;
   if (!(D <= kDmax && (D * es) % 16 == 0)) {
     zp_set_error("attention_score: head_dim %d unsupported (need <= %d and a multiple of %d)", D,
                  kDmax, 16 / es);
@@ -473,14 +522,17 @@ extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
 #define ZP_SCORE_LAUNCH()                                                                        \
   do {                                                                                           \
     const size_t smem = 2 * (size_t)Mma<T>::TN * Mma<T>::ROWB +                                  \
-                        sizeof(float) * (kWaves * Mma<T>::TN) + sizeof(int) * 2 * NB;            \
+                        sizeof(float) * (2 * kRowWaves * Mma<T>::TN + kWaves * 32) + sizeof(int) * 2 * NB;            \
     if (smem > 64 * 1024 &&                                                                      \
-        hipFuncSetAttribute((const void*)score_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                            (int)smem) != hipSuccess) {                                          \
+        (hipFuncSetAttribute((const void*)score_kernel<T, false>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                            (int)smem) != hipSuccess ||                                         \
+         hipFuncSetAttribute((const void*)score_kernel<T, true>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                            (int)smem) != hipSuccess)) {                                          \
       zp_set_error("attention_score: cannot reserve %zu bytes of LDS", smem);                    \
       return ZP_EHIP;                                                                            \
     }                                                                                            \
-    hipLaunchKernelGGL((score_kernel<T>), grid, dim3(kThreads), smem, st, a);                    \
+    if (logits_out) hipLaunchKernelGGL((score_kernel<T, true>), grid, dim3(kThreads), smem, st, a);  \
+    else hipLaunchKernelGGL((score_kernel<T, false>), grid, dim3(kThreads), smem, st, a);        \
   } while (0)
   ZP_DISPATCH_DTYPE(dtype, ZP_SCORE_LAUNCH());
 #undef ZP_SCORE_LAUNCH
