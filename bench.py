@@ -20,6 +20,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes one compaction launch moves per (sequence, layer), from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE scaled by a plain copy kernel (profiles/pipeline_cfg2_b64.md)
+COMPACT_TRAFFIC_PER_SEQ_LAYER = 16_797_469
 
 
 def cpu_baseline(wl, cfg, sample_seqs, budget_s=30.0):
@@ -70,6 +73,13 @@ def main():
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", type=int, default=64)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (read 1 GiB, write 1 GiB) so that a "
+                         "rocprofv3 --pmc run of this command has a kernel of known traffic to "
+                         "scale FETCH_SIZE / WRITE_SIZE by")
+    ap.add_argument("--traffic", type=float, default=None,
+                    help="HBM bytes per compaction launch measured with rocprofv3 --pmc "
+                         "(reported as roofline.traffic)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures the single-GPU hot path only; run with --gpus 1 "
@@ -91,6 +101,14 @@ def main():
     def step(timer=None):
         compress_layers(wl.k, wl.v, wl.q, wl.score_cache, wl.query_ids, wl.block_tables,
                         wl.compressed, wl.targets, cfg, timer=timer)
+
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)  # one streaming kernel: reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step()
@@ -125,7 +143,9 @@ def main():
                    "batch": wl.B, "layers": wl.L},
         "roofline": {"bound": "hbm", "kernel": "compact_kernel (compress_kv)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": args.traffic if args.traffic is not None
+                     else COMPACT_TRAFFIC_PER_SEQ_LAYER * wl.B * wl.L,
                      "algorithmic_bytes": alg["compress_kv"],
                      "avg_launch_us": round(kv_s * 1e6, 2)},
         "pipeline": {"algorithmic_bytes": alg["pipeline"],
