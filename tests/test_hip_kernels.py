@@ -300,7 +300,7 @@ def test_lightning_redundancy(dev, dtype, thr):
     else:
         # a fully claimed row sums to exactly 0 in the oracle and to fp32 noise of a
         # ~200-large cancelling sum here: absolute floor
-        _ulp_close(gl, wl, dtype, ulps=1, frac_exact=0.97, abs_floor=1e-3)
+        _ulp_close(gl, wl, dtype, ulps=1, frac_exact=0.97, abs_floor=1e-2)
         _ulp_close(gr, wr, dtype, ulps=2, frac_exact=0.9)
 
 

@@ -26,6 +26,7 @@ constexpr int ROWF = kDmax + 2;         // floats per LDS row (bank-conflict-fre
 constexpr int KS = kDmax / 2;           // MFMA k-steps (2 per instruction)
 
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 template <typename T> struct Unpack;
 template <> struct Unpack<F32> {
@@ -266,6 +267,405 @@ __global__ __launch_bounds__(kThreads) void gram_kernel(GramArgs p) {
   }
 }
 
+// ------------------------------------------------------------------ 16-bit caches: split-bf16 Gram
+// Same algorithm with the contraction on the bf16 matrix cores.  The fp32 normalised key
+// x = k / n is split into hi = bf16(x) and lo = bf16(x - hi); S = hi.hi + hi.lo + lo.hi drops
+// only the lo.lo term (relative 2^-18), i.e. fp32-grade dot products at a third of the bf16
+// MFMA rate instead of the 16x slower fp32 MFMA.
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+constexpr int ROWH = kDmax * 2 + 16;  // bytes per LDS row of one bf16 plane (16 B pad)
+
+__device__ __forceinline__ void split8(const float* x, bf16x8_t& hi, bf16x8_t& lo) {
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    const __bf16 h = (__bf16)x[q];
+    hi[q] = h;
+    lo[q] = (__bf16)(x[q] - (float)h);
+  }
+}
+
+template <typename T, bool RAW>
+__global__ __launch_bounds__(kThreads, 2) void gram_split_kernel(GramArgs p) {
+  static_assert(T::bytes == 2, "split path is for 16-bit caches");
+  constexpr int PIECES = kDmax / 8;                 // 16-byte pieces per full key row
+  constexpr int ROWS_PER_IT = kThreads / PIECES;    // 16
+  constexpr int STAGE_IT = TN / ROWS_PER_IT;        // 4
+  constexpr int NSUB = TN / 32;
+  constexpr int KSB = kDmax / 16;                   // bf16 MFMA k-steps
+  constexpr int PLANE = TN * ROWH;                  // bytes of one plane of one buffer
+
+  extern __shared__ __align__(16) char smem[];
+  char* buf0 = smem;                                // [hi plane][lo plane]
+  char* buf1 = smem + 2 * PLANE;
+  float* l_sum = (float*)(smem + 4 * PLANE);
+  float* l_val = l_sum + (RAW ? 0 : p.BS);
+  int* l_col = (int*)(l_val + (RAW ? 0 : p.BS));
+  int* vpage = l_col + (RAW ? 0 : p.BS);
+  int* vidx = vpage + p.NB;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const int jp = blockIdx.x % p.NB;
+  const int h = (blockIdx.x / p.NB) % p.Hkv;
+  const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
+  const int l = blockIdx.x / (p.NB * p.Hkv * p.B);
+  const int Tn = p.NB * p.BS;
+  const int64_t orow = (((int64_t)l * p.B + b) * p.Hkv + h);
+  const float epsr = Elem<T>::rnd(p.eps);
+
+  const int code = p.table[(int64_t)b * p.NB + jp];
+  int rpid = page_is_pad(code) ? -1 : page_id(code);
+  if (rpid >= p.num_pages) rpid = -1;
+  if (rpid < 0) {
+    if (!RAW)
+      for (int s = tid; s < p.BS; s += kThreads)
+        Elem<T>::st(p.r_out, orow * Tn + (int64_t)jp * p.BS + s, -INFINITY);
+    return;
+  }
+  __shared__ int ncols_s;
+  if (tid == 0) {
+    int n = 0;
+    if (RAW) {
+      for (int j = 0; j < p.NB; ++j) {
+        const int c = p.table[(int64_t)b * p.NB + j];
+        const int pid = page_is_pad(c) ? -1 : page_id(c);
+        if (pid >= 0 && pid < p.num_pages) { vpage[n] = pid; vidx[n] = j; ++n; }
+      }
+    } else {
+      vpage[0] = rpid; vidx[0] = jp; n = 1;
+    }
+    ncols_s = n;
+  }
+  for (int i = tid; i < 4 * PLANE / 4; i += kThreads) ((uint32_t*)smem)[i] = 0u;
+  __syncthreads();
+  const int tiles_per_page = p.BS / TN;
+  const int ntiles = ncols_s * tiles_per_page;
+  const int dpieces = p.D / 8;
+  const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
+  const char* kbase = p.k + (l * p.k_sl) * 2 + (int64_t)h * p.D * 2;
+
+  const int st_piece = tid % PIECES, st_row0 = tid / PIECES;
+  vec16 pre[STAGE_IT];
+  auto issue_loads = [&](int tile) {
+    const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
+    const char* src = kbase + (int64_t)vpage[vp] * p.k_sp * 2 + (int64_t)toff * k_row;
+#pragma unroll
+    for (int i = 0; i < STAGE_IT; ++i) {
+      const int row = st_row0 + i * ROWS_PER_IT;
+      const int pc = st_piece < dpieces ? st_piece : 0;  // clamp: unconditional load
+      pre[i] = *(const vec16*)(src + (int64_t)row * k_row + pc * 16);
+    }
+  };
+  auto commit_loads = [&](char* buf) {
+#pragma unroll
+    for (int i = 0; i < STAGE_IT; ++i) {
+      const int row = st_row0 + i * ROWS_PER_IT;
+      float e[8];
+      Unpack<T>::run(pre[i], e);
+      float ss = 0.f;
+      if (st_piece < dpieces) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) ss += e[q] * e[q];
+      }
+#pragma unroll
+      for (int o = PIECES >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      const float n = fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
+      if (st_piece < dpieces) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) e[q] = e[q] / n;
+        bf16x8_t hi, lo;
+        split8(e, hi, lo);
+        *(bf16x8_t*)(buf + row * ROWH + st_piece * 16) = hi;
+        *(bf16x8_t*)(buf + PLANE + row * ROWH + st_piece * 16) = lo;
+      }
+    }
+  };
+
+  const int row_blocks = p.BS / 32;
+  const int NR = (row_blocks + kWaves - 1) / kWaves;
+  for (int rr = 0; rr < NR; ++rr) {
+    const int rb = rr * kWaves + wave;
+    const bool active = rb < row_blocks;
+    // ---- A fragments: this lane's key row; lane (row, half) holds k = 16 s + 8 half + i
+    bf16x8_t ahi[KSB], alo[KSB];
+    {
+      const int slot = (active ? rb : 0) * 32 + col;
+      const char* src = kbase + (int64_t)rpid * p.k_sp * 2 + (int64_t)slot * k_row;
+      float x[KSB][8];
+      float ss = 0.f;
+#pragma unroll
+      for (int s = 0; s < KSB; ++s) {
+        const int pc = 2 * s + half;
+        vec16 v = vec16{0u, 0u, 0u, 0u};
+        if (pc < dpieces) v = *(const vec16*)(src + pc * 16);
+        Unpack<T>::run(v, x[s]);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) ss += x[s][q] * x[s][q];
+      }
+      ss += __shfl_xor(ss, 32, 64);  // the other half of the row
+      const float n = fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
+#pragma unroll
+      for (int s = 0; s < KSB; ++s) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) x[s][q] = active ? x[s][q] / n : 0.f;
+        split8(x[s], ahi[s], alo[s]);
+      }
+    }
+    float rsum[16], cval[16];
+    int ccol[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { rsum[r] = 0.f; cval[r] = 0.f; ccol[r] = -1; }
+
+    if (ntiles > 0) { issue_loads(0); commit_loads(buf0); }
+    __syncthreads();
+    for (int tile = 0; tile < ntiles; ++tile) {
+      char* cur = (tile & 1) ? buf1 : buf0;
+      char* nxt = (tile & 1) ? buf0 : buf1;
+      if (tile + 1 < ntiles) issue_loads(tile + 1);
+      const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
+      const int jc = vidx[vp];
+      if (active) {
+#pragma unroll 1
+        for (int st = 0; st < NSUB; ++st) {
+          f32x16_t acc;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+          const char* brow = cur + (st * 32 + col) * ROWH + half * 16;
+#pragma unroll
+          for (int s0 = 0; s0 < KSB; s0 += 4) {
+            bf16x8_t bh[4], bl[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+              bh[s] = *(const bf16x8_t*)(brow + (s0 + s) * 32);
+              bl[s] = *(const bf16x8_t*)(brow + PLANE + (s0 + s) * 32);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[s0 + s], bh[s], acc, 0, 0, 0);
+              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[s0 + s], bl[s], acc, 0, 0, 0);
+              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo[s0 + s], bh[s], acc, 0, 0, 0);
+            }
+          }
+          const int cslot = toff + st * 32 + col;
+          const int cidx = jc * p.BS + cslot;
+          const bool same_page = jc == jp;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+            float s = acc[r];
+            if (same_page && rslot == cslot) s = 0.f;
+            rsum[r] += s;
+            if (s > p.threshold) { ccol[r] = cidx; cval[r] = s; }
+          }
+        }
+      }
+      if (tile + 1 < ntiles) commit_loads(nxt);
+      __syncthreads();
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float s = rsum[r];
+      int c = ccol[r];
+      float v = cval[r];
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) {
+        s += __shfl_xor(s, o, 64);
+        const int oc = __shfl_xor(c, o, 64);
+        const float ov = __shfl_xor(v, o, 64);
+        if (oc > c) { c = oc; v = ov; }
+      }
+      if (active && col == 0) {
+        const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+        if (RAW) {
+          const int64_t oi = orow * Tn + (int64_t)jp * p.BS + rslot;
+          p.ws_sum[oi] = s;
+          p.ws_col[oi] = c;
+          p.ws_val[oi] = v;
+        } else {
+          l_sum[rslot] = s;
+          l_col[rslot] = c - jp * p.BS;
+          l_val[rslot] = v;
+        }
+      }
+    }
+  }
+  if (!RAW) {
+    __syncthreads();
+    for (int i = tid; i < p.BS; i += kThreads) {
+      float corr = 0.f;
+      for (int j = 0; j < p.BS; ++j)
+        if (l_col[j] == i) corr += l_val[j];
+      Elem<T>::st(p.r_out, orow * Tn + (int64_t)jp * p.BS + i, l_sum[i] - corr);
+    }
+  }
+}
+
+// ------------------------------------------------------------------ lightning, whole page in LDS
+// Per-page variant for 16-bit caches and pages of up to 256 keys: the page is normalised and
+// split once into LDS (hi and lo planes, 2 x 68 KB), after which eight waves each own a
+// 32-row block and run over all column blocks with no further staging or barriers.
+constexpr int kPageThreads = 512;
+constexpr int kPageRows = 256;
+
+template <typename T>
+__global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
+  static_assert(T::bytes == 2, "16-bit caches only");
+  constexpr int PIECES = kDmax / 8;
+  constexpr int KSB = kDmax / 16;
+  constexpr int PLANE = kPageRows * ROWH;
+
+  extern __shared__ __align__(16) char smem[];
+  char* hi_pl = smem;
+  char* lo_pl = smem + PLANE;
+  float* l_sum = (float*)(smem + 2 * PLANE);
+  float* l_val = l_sum + kPageRows;
+  int* l_col = (int*)(l_val + kPageRows);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const int jp = blockIdx.x % p.NB;
+  const int h = (blockIdx.x / p.NB) % p.Hkv;
+  const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
+  const int l = blockIdx.x / (p.NB * p.Hkv * p.B);
+  const int Tn = p.NB * p.BS;
+  const int64_t obase = (((int64_t)l * p.B + b) * p.Hkv + h) * Tn + (int64_t)jp * p.BS;
+  const float epsr = Elem<T>::rnd(p.eps);
+
+  const int code = p.table[(int64_t)b * p.NB + jp];
+  int rpid = page_is_pad(code) ? -1 : page_id(code);
+  if (rpid >= p.num_pages) rpid = -1;
+  if (rpid < 0) {
+    for (int s = tid; s < p.BS; s += kPageThreads) Elem<T>::st(p.r_out, obase + s, -INFINITY);
+    return;
+  }
+  const int dpieces = p.D / 8;
+  const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
+  const char* page = p.k + (l * p.k_sl + (int64_t)rpid * p.k_sp) * 2 + (int64_t)h * p.D * 2;
+
+  // ---- stage: normalise and split every key of the page
+  {
+    const int piece = tid % PIECES, row0 = tid / PIECES;       // 32 rows per iteration
+    constexpr int ROWS_PER_IT = kPageThreads / PIECES;
+    constexpr int ITERS = kPageRows / ROWS_PER_IT;
+    // all loads of the page are in flight before the first one is consumed
+    u32x4 raw[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int row = it * ROWS_PER_IT + row0;
+      raw[it] = *(const u32x4*)(page + (int64_t)(row < p.BS ? row : 0) * k_row +
+                                (piece < dpieces ? piece : 0) * 16);
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int row = it * ROWS_PER_IT + row0;
+      const bool ok = row < p.BS && piece < dpieces;
+      const vec16 v = vec16{raw[it].x, raw[it].y, raw[it].z, raw[it].w};
+      float e[8];
+      Unpack<T>::run(v, e);
+      float ss = 0.f;
+      if (ok) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) ss += e[q] * e[q];
+      }
+#pragma unroll
+      for (int o = PIECES >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      const float rn = 1.f / fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
+      bf16x8_t hi, lo;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) e[q] = ok ? e[q] * rn : 0.f;
+      split8(e, hi, lo);
+      if (row < p.BS) {
+        *(bf16x8_t*)(hi_pl + row * ROWH + piece * 16) = hi;
+        *(bf16x8_t*)(lo_pl + row * ROWH + piece * 16) = lo;
+      }
+    }
+  }
+  __syncthreads();
+
+  const int row_blocks = p.BS / 32;
+  for (int rb = wave; rb < row_blocks; rb += kPageThreads / 64) {
+    bf16x8_t ahi[KSB], alo[KSB];
+    {
+      const char* arow = hi_pl + (rb * 32 + col) * ROWH + half * 16;
+#pragma unroll
+      for (int s = 0; s < KSB; ++s) {
+        ahi[s] = *(const bf16x8_t*)(arow + s * 32);
+        alo[s] = *(const bf16x8_t*)(arow + PLANE + s * 32);
+      }
+    }
+    float rsum[16], cval[16];
+    int ccol[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { rsum[r] = 0.f; cval[r] = 0.f; ccol[r] = -1; }
+#pragma unroll 1
+    for (int cb = 0; cb < row_blocks; ++cb) {
+      f32x16_t acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+      const char* brow = hi_pl + (cb * 32 + col) * ROWH + half * 16;
+#pragma unroll
+      for (int s0 = 0; s0 < KSB; s0 += 4) {
+        bf16x8_t bh[4], bl[4];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          bh[s] = *(const bf16x8_t*)(brow + (s0 + s) * 32);
+          bl[s] = *(const bf16x8_t*)(brow + PLANE + (s0 + s) * 32);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[s0 + s], bh[s], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[s0 + s], bl[s], acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo[s0 + s], bh[s], acc, 0, 0, 0);
+        }
+      }
+      const int cslot = cb * 32 + col;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+        float s = acc[r];
+        if (rslot == cslot) s = 0.f;
+        rsum[r] += s;
+        if (s > p.threshold) { ccol[r] = cslot; cval[r] = s; }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float s = rsum[r];
+      int c = ccol[r];
+      float v = cval[r];
+#pragma unroll
+      for (int o = 16; o > 0; o >>= 1) {
+        s += __shfl_xor(s, o, 64);
+        const int oc = __shfl_xor(c, o, 64);
+        const float ov = __shfl_xor(v, o, 64);
+        if (oc > c) { c = oc; v = ov; }
+      }
+      if (col == 0) {
+        const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+        l_sum[rslot] = s;
+        l_col[rslot] = c;
+        l_val[rslot] = v;
+      }
+    }
+  }
+  __syncthreads();
+  // r_i = rowsum_i - sum of the entries other rows claimed from row i (ascending j: deterministic)
+  for (int i = tid; i < p.BS; i += kPageThreads) {
+    float corr = 0.f;
+    for (int j = 0; j < p.BS; j += 4) {
+      const int4 c4 = *(const int4*)(l_col + j);
+      const float4 v4 = *(const float4*)(l_val + j);
+      if (c4.x == i) corr += v4.x;
+      if (c4.y == i) corr += v4.y;
+      if (c4.z == i) corr += v4.z;
+      if (c4.w == i) corr += v4.w;
+    }
+    Elem<T>::st(p.r_out, obase + i, l_sum[i] - corr);
+  }
+}
+
 // ------------------------------------------------------------------ softmax epilogue
 // One workgroup per (layer, sequence, head) row of T logits:
 //   raw only: r_i = rowsum_i - sum_{j: c*(j)=i} v_j, pad pages -inf
@@ -370,16 +770,40 @@ int check_common(const char* name, const void* k_cache, const int32_t* table, vo
 
 template <typename T, bool RAW>
 int launch_gram(const GramArgs& a, int L, hipStream_t st) {
-  const size_t smem = sizeof(float) * 2 * TN * ROWF + (RAW ? 0 : (size_t)a.BS * 12) +
-                      sizeof(int) * 2 * a.NB;
-  if (smem > 64 * 1024 &&
-      hipFuncSetAttribute((const void*)gram_kernel<T, RAW>,
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
-    zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
-    return ZP_EHIP;
-  }
   dim3 grid((unsigned)((int64_t)L * a.B * a.Hkv * a.NB));
-  hipLaunchKernelGGL((gram_kernel<T, RAW>), grid, dim3(kThreads), smem, st, a);
+  const size_t tail = (RAW ? 0 : (size_t)a.BS * 12) + sizeof(int) * 2 * a.NB;
+  if constexpr (T::bytes == 2 && !RAW) {
+    if (a.BS <= kPageRows && a.BS % 32 == 0) {
+      const size_t smem = 2 * (size_t)kPageRows * ROWH + (size_t)kPageRows * 12;
+      if (hipFuncSetAttribute((const void*)gram_page_kernel<T>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+        zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
+        return ZP_EHIP;
+      }
+      hipLaunchKernelGGL((gram_page_kernel<T>), grid, dim3(kPageThreads), smem, st, a);
+      ZP_LAUNCH_CHECK();
+      return ZP_OK;
+    }
+  }
+  if constexpr (T::bytes == 2) {
+    const size_t smem = 4 * (size_t)TN * ROWH + tail;
+    if (smem > 64 * 1024 &&
+        hipFuncSetAttribute((const void*)gram_split_kernel<T, RAW>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+      zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
+      return ZP_EHIP;
+    }
+    hipLaunchKernelGGL((gram_split_kernel<T, RAW>), grid, dim3(kThreads), smem, st, a);
+  } else {
+    const size_t smem = sizeof(float) * 2 * TN * ROWF + tail;
+    if (smem > 64 * 1024 &&
+        hipFuncSetAttribute((const void*)gram_kernel<T, RAW>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+      zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
+      return ZP_EHIP;
+    }
+    hipLaunchKernelGGL((gram_kernel<T, RAW>), grid, dim3(kThreads), smem, st, a);
+  }
   ZP_LAUNCH_CHECK();
   return ZP_OK;
 }

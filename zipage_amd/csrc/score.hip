@@ -27,8 +27,11 @@
 
 namespace {
 
-constexpr int kThreads = 512;
-constexpr int kWaves = 8;      // waves per workgroup
+#ifndef ZP_SCORE_WAVES
+#define ZP_SCORE_WAVES 8
+#endif
+constexpr int kWaves = ZP_SCORE_WAVES;  // waves per workgroup (4 or 8)
+constexpr int kThreads = kWaves * 64;
 constexpr int kRowWaves = 4;   // waves along the query-row axis; the other factor splits tokens
 constexpr int kTokWaves = kWaves / kRowWaves;
 constexpr int kDmax = 128;
@@ -40,21 +43,21 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 template <typename T> struct Mma;
 template <> struct Mma<BF16> {
   typedef bf16x8_t Frag;
-  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = 256, ROWB = kDmax * 2 + 16;
+  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = 32 * kWaves, ROWB = kDmax * 2 + 16;
   __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
 };
 template <> struct Mma<F16> {
   typedef f16x8_t Frag;
-  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = 256, ROWB = kDmax * 2 + 16;
+  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = 32 * kWaves, ROWB = kDmax * 2 + 16;
   __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
 };
 template <> struct Mma<F32> {
   typedef float Frag;
-  static constexpr int KPI = 2, EPL = 1, KS = kDmax / KPI, TN = 128, ROWB = kDmax * 4 + 8;
+  static constexpr int KPI = 2, EPL = 1, KS = kDmax / KPI, TN = 16 * kWaves, ROWB = kDmax * 4 + 8;
   __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
   }
@@ -117,7 +120,7 @@ __device__ __forceinline__ float exp_neg(float x) {
 }
 
 template <typename T, bool LOGITS>
-__global__ __launch_bounds__(kThreads) void score_kernel(ScoreArgs p) {
+__global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? 2 : 1)) void score_kernel(ScoreArgs p) {
   typedef Mma<T> M;
   typedef typename M::Frag Frag;
   constexpr int TN = M::TN, NSUB = TN / 32 / kTokWaves, ROWB = M::ROWB, KS = M::KS;
@@ -481,7 +484,7 @@ extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
              "attention_score: unknown reduction %d", reduced);
   ZP_REQUIRE(W <= BS, "attention_score: window %d longer than a page of %d", W, BS);
   const int es = zp_dtype_bytes(dtype);
-  const int TN = dtype == ZP_F32 ? 128 : 256;
+  const int TN = dtype == ZP_F32 ? Mma<F32>::TN : Mma<BF16>::TN;
   if (!(D <= kDmax && (D * es) % 16 == 0)) {
     zp_set_error("attention_score: head_dim %d unsupported (need <= %d and a multiple of %d)", D,
                  kDmax, 16 / es);
