@@ -651,18 +651,34 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
     }
   }
   __syncthreads();
-  // r_i = rowsum_i - sum of the entries other rows claimed from row i (ascending j: deterministic)
-  for (int i = tid; i < p.BS; i += kPageThreads) {
+  // r_i = rowsum_i - sum of the entries other rows claimed from row i.  Claims usually land on
+  // a few rows, so a presence mask lets every other row skip the scan; two threads share a row
+  // (fixed split and order: deterministic sums).
+  __shared__ uint32_t claimed[kPageRows / 32];
+  if (tid < kPageRows / 32) claimed[tid] = 0u;
+  __syncthreads();
+  if (tid < p.BS) {
+    const int c = l_col[tid];
+    if (c >= 0) atomicOr(&claimed[c >> 5], 1u << (c & 31));
+  }
+  __syncthreads();
+  {
+    const int i = tid >> 1, part = tid & 1;
     float corr = 0.f;
-    for (int j = 0; j < p.BS; j += 4) {
-      const int4 c4 = *(const int4*)(l_col + j);
-      const float4 v4 = *(const float4*)(l_val + j);
-      if (c4.x == i) corr += v4.x;
-      if (c4.y == i) corr += v4.y;
-      if (c4.z == i) corr += v4.z;
-      if (c4.w == i) corr += v4.w;
+    const bool need = i < p.BS && ((claimed[i >> 5] >> (i & 31)) & 1u);
+    if (need) {
+      const int j0 = part * (kPageRows / 2);
+      for (int j = j0; j < j0 + kPageRows / 2 && j < p.BS; j += 4) {
+        const int4 c4 = *(const int4*)(l_col + j);
+        const float4 v4 = *(const float4*)(l_val + j);
+        if (c4.x == i) corr += v4.x;
+        if (c4.y == i) corr += v4.y;
+        if (c4.z == i) corr += v4.z;
+        if (c4.w == i) corr += v4.w;
+      }
     }
-    Elem<T>::st(p.r_out, obase + i, l_sum[i] - corr);
+    const float other = __shfl_xor(corr, 1, 64);
+    if (part == 0 && i < p.BS) Elem<T>::st(p.r_out, obase + i, l_sum[i] - (corr + other));
   }
 }
 

@@ -32,8 +32,9 @@ namespace {
 #endif
 constexpr int kWaves = ZP_SCORE_WAVES;  // waves per workgroup (4 or 8)
 constexpr int kThreads = kWaves * 64;
-constexpr int kRowWaves = 4;   // waves along the query-row axis; the other factor splits tokens
-constexpr int kTokWaves = kWaves / kRowWaves;
+constexpr int kRowWaves = 4;   // most waves along the query-row axis; the other factor splits tokens.
+                               // Fewer row blocks (small window x group) use 2 or 1 row waves so
+                               // that no wave idles: ScoreArgs::RW.
 constexpr int kDmax = 128;
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -77,6 +78,7 @@ struct ScoreArgs {
   int reduce_max;
   int RB;  // row blocks of 32
   int gs;  // log2(Gp)
+  int RW;  // waves along the row axis: 1, 2 or 4
 };
 
 template <typename T>
@@ -123,7 +125,9 @@ template <typename T, bool LOGITS>
 __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? 2 : 1)) void score_kernel(ScoreArgs p) {
   typedef Mma<T> M;
   typedef typename M::Frag Frag;
-  constexpr int TN = M::TN, NSUB = TN / 32 / kTokWaves, ROWB = M::ROWB, KS = M::KS;
+  constexpr int TN = M::TN, ROWB = M::ROWB, KS = M::KS;
+  const int RW = p.RW, TW = kWaves / RW;  // row waves x token waves
+  const int NSUB = TN / 32 / TW;          // subtiles per wave and tile
   constexpr int PIECES = kDmax * T::bytes / 16;       // 16-byte pieces per full key row
   constexpr int ROWS_PER_IT = kThreads / PIECES;      // rows staged per iteration
   constexpr int STAGE_IT = TN / ROWS_PER_IT;          // iterations (== 8)
@@ -138,7 +142,7 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? 2 : 1)) v
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
-  const int rbw = wave % kRowWaves, tg = wave / kRowWaves;  // row-block wave, token group
+  const int rbw = wave % RW, tg = wave / RW;  // row-block wave, token group
   const int h = blockIdx.x % p.Hkv;
   const int b = (blockIdx.x / p.Hkv) % p.B;
   const int l = blockIdx.x / (p.Hkv * p.B);
@@ -213,11 +217,11 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? 2 : 1)) v
     }
   };
 
-  const int NR = (p.RB + kRowWaves - 1) / kRowWaves;  // row rounds
+  const int NR = (p.RB + RW - 1) / RW;  // row rounds
   const float ascale = fabsf(p.scale);
   const float sgn = p.scale < 0.f ? -1.f : 1.f;
   for (int rr = 0; rr < NR; ++rr) {
-    const int rb = rr * kRowWaves + rbw;
+    const int rb = rr * RW + rbw;
     const bool active = rb < p.RB;
     // ---- A fragments: query rows of this wave's row block
     Frag afrag[KS];
@@ -252,7 +256,7 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? 2 : 1)) v
           const float* pt = part + (tile & 1) * kRowWaves * TN;
           float v = pt[tid];
 #pragma unroll
-          for (int w2 = 1; w2 < kRowWaves; ++w2)
+          for (int w2 = 1; w2 < RW; ++w2)
             v = p.reduce_max ? fmaxf(v, pt[w2 * TN + tid]) : v + pt[w2 * TN + tid];
           const int64_t oi = orow * Tn + (int64_t)j * p.BS + toff + tid;
           if (NR > 1) {
@@ -424,8 +428,8 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? 2 : 1)) v
         for (int r = 0; r < 16; ++r) {
           float v = run[r];
 #pragma unroll
-          for (int g2 = 1; g2 < kTokWaves; ++g2) {
-            const int ow = ((tg + g2) % kTokWaves) * kRowWaves + rbw;
+          for (int g2 = 1; g2 < TW; ++g2) {
+            const int ow = ((tg + g2) % TW) * RW + rbw;
             const float t = stat[ow * 32 + (r >> 2) * 8 + half * 4 + (r & 3)];
             v = PASS == 0 ? fmaxf(v, t) : v + t;
           }
@@ -519,6 +523,8 @@ extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
   a.scale = softmax_scale; a.reduce_max = reduced == ZP_REDUCE_MAX; a.RB = RB;
   a.gs = 0;
   while ((1 << a.gs) < Gp) ++a.gs;
+  a.RW = RB >= 3 ? kRowWaves : RB;
+  if (a.RW < kWaves / (TN / 32)) a.RW = kWaves / (TN / 32);  // every wave needs >= 1 subtile
 
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned)((int64_t)L * B * Hkv));
