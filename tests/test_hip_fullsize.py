@@ -1,0 +1,187 @@
+"""GPU checks at the BASELINE sizes, where the CPU oracle is too slow for the whole batch:
+size-independent properties over every sequence, plus the oracle on a sample of sequences.
+
+Properties (each row = one (layer, sequence, kv head)):
+  * exactly k = 2048 keep flags per row, none on padding pages, all window slots kept;
+  * the flags are what the oracle selector picks from the GPU's own scores (lowest index wins);
+  * compaction is a stable gather: the kept (page, slot) vectors of K and V, read BEFORE the
+    call, equal the target pages read AFTER it, in order, bit for bit;
+  * read-only shared-prefix pages are untouched;
+  * running the compaction again with "keep everything that is now in the budget" is the
+    identity (idempotence).
+"""
+import pytest
+import torch
+
+from oracle import zipage_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+BS, BUDGET = 256, 8
+
+
+def _run_pipeline(wl, cfg):
+    from zipage_amd.compress import compress_layers
+    return compress_layers(wl.k, wl.v, wl.q, wl.score_cache, wl.query_ids, wl.block_tables,
+                           wl.compressed, wl.targets, cfg, return_intermediates=True)
+
+
+def _gather_rows(cache, tables_enc, flag_or_none, l=0):
+    """(B, Hkv) lists are too slow at this size; return a dense gather instead:
+    pages (B, NB) -> tensor (B, NB*BS, Hkv, D) with padding pages zero-filled."""
+    B, NB = tables_enc.shape
+    pid = torch.where(tables_enc < -1, -tables_enc - 2, tables_enc).clamp(min=0).long()
+    out = cache[l][pid.flatten()].view(B, NB * BS, *cache.shape[-2:])
+    return out
+
+
+def _check_properties(wl, flag, scores, k_before, v_before, shared_pages=()):
+    L, B, Hkv, NB, _ = flag.shape
+    T = NB * BS
+    kk = BUDGET * BS
+    f = flag.view(L, B, Hkv, T)
+    assert (f.sum(-1) == kk).all(), "every row keeps exactly k tokens"
+    pad = (wl.block_tables == -1)
+    assert not (flag & pad.view(1, B, 1, NB, 1)).any(), "padding pages are never kept"
+    last = (wl.block_tables < -1).view(1, B, 1, NB, 1).expand_as(flag)
+    win = torch.zeros_like(flag)
+    win[..., BS - wl.W:] = True
+    assert flag[last & win].all(), "the window slots of the last page are always kept"
+    # selector against the oracle on the GPU's own scores
+    want = O.topk_mask(scores.cpu().view(L, B, Hkv, T), kk)
+    assert torch.equal(f.cpu(), want)
+    # stable gather, checked densely on the device for layer 0
+    enc = wl.block_tables
+    src_k = _gather_rows(k_before, enc, None)          # (B, T, Hkv, D) from the saved copy
+    src_v = _gather_rows(v_before, enc, None)
+    tgt = wl.targets[:, :BUDGET].long()
+    got_k = wl.k[0][tgt.flatten()].view(B, kk, Hkv, -1)
+    got_v = wl.v[0][tgt.flatten()].view(B, kk, Hkv, -1)
+    for h in range(Hkv):
+        keep = f[0, :, h]                               # (B, T)
+        order = torch.argsort((~keep).to(torch.int8), dim=1, stable=True)[:, :kk]  # kept, ascending
+        idx = order.unsqueeze(-1).expand(B, kk, src_k.shape[-1])
+        assert torch.equal(got_k[:, :, h], torch.gather(src_k[:, :, h], 1, idx))
+        assert torch.equal(got_v[:, :, h], torch.gather(src_v[:, :, h], 1, idx))
+    for p in shared_pages:
+        assert torch.equal(wl.k[0, p], k_before[0, p]) and torch.equal(wl.v[0, p], v_before[0, p])
+
+
+def _save_touched(wl):
+    """Copies of K and V restricted to the touched pages, addressable by original page id
+    through a sparse clone (untouched pages are never read by the checks)."""
+    pages = sorted({p for t in wl.tables for p in t} | set(wl.targets.flatten().tolist()))
+    idx = torch.tensor(pages, device=wl.k.device)
+    kb = torch.empty_like(wl.k)
+    vb = torch.empty_like(wl.v)
+    kb[:, idx] = wl.k[:, idx]
+    vb[:, idx] = wl.v[:, idx]
+    return kb, vb
+
+
+def _oracle_sample(wl, sub, cfg_kwargs, seq_ids, scores_gpu, dtype):
+    """`sub` = cpu_subset(wl, seq_ids) taken BEFORE the in-place pipeline ran."""
+    s = O.attention_score(sub["k"], sub["q"], sub["query_ids"], sub["block_tables"])
+    if cfg_kwargs.get("enable_pooling"):
+        s = O.pool_scores(s, sub["compressed"], cfg_kwargs.get("pooling_size", 5))
+    s = O.pad_mask(O.window_mask(s, sub["block_tables"], wl.W), sub["block_tables"])
+    g = scores_gpu[:, seq_ids].float().cpu()
+    w = s.float()
+    assert torch.equal(torch.isinf(g), torch.isinf(w))
+    fin = torch.isfinite(w)
+    rel = 1e-3 if dtype == torch.float32 else 2.0 ** -6
+    bad = ((g[fin] - w[fin]).abs() > rel * w[fin].abs() + 1e-9).float().mean().item()
+    assert bad <= (0.0 if dtype == torch.float32 else 2e-3), f"{bad} of sampled scores off"
+
+
+def test_config2_64_ragged_sequences(dev):
+    """BASELINE configs[1]: 64 sequences, Qwen3-8B shape, bf16, 20k-page pool."""
+    from zipage_amd.compress import CompressConfig
+    from zipage_amd.workload import cpu_subset, ragged_batch
+    wl = ragged_batch(64, L=1, pool_pages=20000, budget=BUDGET, W=32, seed=1, lengths=(2049, 2304))
+    kb, vb = _save_touched(wl)
+    sub = cpu_subset(wl, [0, 17, 63])
+    kw = dict(enable_pooling=True, pooling_size=7)
+    cfg = CompressConfig(budget_blocks=BUDGET, query_cache_len=32, **kw)
+    flag, scores = _run_pipeline(wl, cfg)
+    _check_properties(wl, flag, scores, kb, vb)
+    _oracle_sample(wl, sub, kw, [0, 17, 63], scores, torch.bfloat16)
+    # idempotence: the survivors now fill pages 0..7 of each target; keeping exactly those
+    # again must not move a byte
+    from zipage_amd.kernel import compress_kv
+    k_after, v_after = _save_touched(wl)
+    B, NB = wl.block_tables.shape
+    keep_all = torch.zeros((1, B, 8, NB, BS), dtype=torch.bool, device=wl.k.device)
+    keep_all[:, :, :, :BUDGET] = True
+    compress_kv(wl.k, wl.v, keep_all, wl.block_tables, wl.targets)
+    idx = torch.tensor(sorted(set(wl.targets.flatten().tolist())), device=wl.k.device)
+    assert torch.equal(wl.k[:, idx], k_after[:, idx]) and torch.equal(wl.v[:, idx], v_after[:, idx])
+
+
+def test_config4_prefix_sharing_copy_on_write(dev):
+    """BASELINE configs[3], one layer: 256 sequences, groups of 16 share their first 2 pages,
+    lengths up to 2560 (9 or 10 pages), 60k-page pool; targets follow the copy-on-write rule so
+    shared pages are read-only sources."""
+    from zipage_amd.compress import CompressConfig
+    from zipage_amd.workload import cpu_subset, ragged_batch
+    wl = ragged_batch(256, L=1, pool_pages=60000, budget=BUDGET, W=32, seed=3, lengths=(2049, 2560),
+                      shared_prefix_group=16, shared_prefix_pages=2)
+    assert wl.block_tables.shape[1] == 10 and (wl.block_tables == -1).any()
+    shared = sorted({t[0] for t in wl.tables} | {t[1] for t in wl.tables})
+    assert len(shared) == 2 * 16
+    kb, vb = _save_touched(wl)
+    sub = cpu_subset(wl, [0, 16, 255])
+    kw = dict(enable_pooling=True, pooling_size=7)
+    cfg = CompressConfig(budget_blocks=BUDGET, query_cache_len=32, **kw)
+    flag, scores = _run_pipeline(wl, cfg)
+    _check_properties(wl, flag, scores, kb, vb, shared_pages=shared)
+    _oracle_sample(wl, sub, kw, [0, 16, 255], scores, torch.bfloat16)
+
+
+def test_config1_single_sequence_fp32_full_oracle(dev):
+    """BASELINE configs[0]: one sequence, Qwen3-0.6B shape (16 q / 8 kv heads), fp32, 9 pages
+    from a 64-page pool, window 32, max-pool 7, keep 2048 -- compared in full with the oracle."""
+    from zipage_amd.compress import CompressConfig
+    from zipage_amd.workload import QWEN3_0_6B, cpu_subset, ragged_batch
+    wl = ragged_batch(1, L=1, pool_pages=64, budget=BUDGET, W=32, seed=0, lengths=(2304, 2304),
+                      dtype=torch.float32, shape=QWEN3_0_6B)
+    sub = cpu_subset(wl, [0])
+    kw = dict(enable_pooling=True, pooling_size=7)
+    oflag, oscores = O.compress_pipeline(
+        sub["k"], sub["v"], sub["q"], None, sub["query_ids"], sub["block_tables"], sub["compressed"],
+        sub["targets"], budget_blocks=BUDGET, query_cache_len=32, return_intermediates=True, **kw)
+    flag, scores = _run_pipeline(wl, CompressConfig(budget_blocks=BUDGET, query_cache_len=32, **kw))
+    g, w = scores.float().cpu(), oscores.float()
+    fin = torch.isfinite(w)
+    assert torch.equal(torch.isinf(g), torch.isinf(w))
+    assert ((g[fin] - w[fin]).abs() <= 1e-3 * w[fin].abs() + 1e-10).all()
+    assert torch.equal(flag.cpu(), O.topk_mask(scores.cpu().view(1, 1, 8, -1), 2048).view_as(flag))
+    mism = (flag.cpu() != oflag).float().mean().item()
+    assert mism <= 1e-3
+    if mism == 0:
+        pages = torch.tensor(sub["pages"], device=wl.k.device)
+        assert torch.equal(wl.k[:, pages].cpu(), sub["k"]) and torch.equal(wl.v[:, pages].cpu(), sub["v"])
+
+
+def test_config3_global_score_and_redundancy_128_sequences(dev):
+    """BASELINE configs[2]: configs[0] shape and dtype, 128 sequences, carried global score
+    (decay 0.9) and lightning redundancy; properties on the batch, oracle on two sequences."""
+    from zipage_amd.compress import CompressConfig
+    from zipage_amd.workload import QWEN3_0_6B, cpu_subset, ragged_batch
+    wl = ragged_batch(128, L=1, pool_pages=2000, budget=BUDGET, W=32, seed=2, lengths=(2304, 2304),
+                      dtype=torch.float32, shape=QWEN3_0_6B, with_score_cache=True, compressed=True)
+    kb, vb = _save_touched(wl)
+    kw = dict(use_global_score=True, decay_factor=0.9, use_redudancy=True, lightning_redudancy=True,
+              redudancy_lambda=0.5, enable_pooling=True, pooling_size=7, continues_pooling=True)
+    ids = [5, 100]
+    sub = cpu_subset(wl, ids)
+    oflag, oscores = O.compress_pipeline(
+        sub["k"], sub["v"], sub["q"], sub["score_cache"], sub["query_ids"], sub["block_tables"],
+        sub["compressed"], sub["targets"], budget_blocks=BUDGET, query_cache_len=32,
+        return_intermediates=True, **kw)
+    flag, scores = _run_pipeline(wl, CompressConfig(budget_blocks=BUDGET, query_cache_len=32, **kw))
+    _check_properties(wl, flag, scores, kb, vb)
+    g, w = scores[:, ids].float().cpu(), oscores.float()
+    fin = torch.isfinite(w)
+    assert torch.equal(torch.isinf(g), torch.isinf(w))
+    assert ((g[fin] - w[fin]).abs() <= 1e-3 * w[fin].abs() + 1e-8).all()

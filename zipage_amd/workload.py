@@ -132,3 +132,26 @@ def algorithmic_bytes(wl: Workload, cfg) -> dict:
         out["redudancy_score"] = L * valid_pages * BS * Hkv * D * es
     out["pipeline"] = sum(out.values())
     return out
+
+
+def cpu_subset(wl: Workload, seq_ids):
+    """Host copy of the sequences ``seq_ids`` with their pages renumbered densely, for checking
+    or timing against a CPU implementation.  Returns a dict of CPU tensors with the same
+    meaning as the Workload fields (block tables already encoded)."""
+    seq_ids = list(seq_ids)
+    tables = [wl.tables[b] for b in seq_ids]
+    targets = wl.targets[seq_ids].tolist()
+    used = sorted({p for t in tables for p in t} | {int(p) for row in targets for p in row})
+    remap = {p: i for i, p in enumerate(used)}
+    idx = torch.tensor(used, device=wl.k.device)
+    width = wl.block_tables.shape[1]
+    rows = [[remap[p] for p in t] for t in tables]
+    enc = torch.tensor([r[:-1] + [-r[-1] - 2] + [-1] * (width - len(r)) for r in rows],
+                       dtype=torch.int32)
+    return dict(
+        k=wl.k[:, idx].cpu(), v=wl.v[:, idx].cpu(), q=wl.q[:, seq_ids].cpu(),
+        score_cache=None if wl.score_cache is None else wl.score_cache[:, idx].cpu(),
+        query_ids=torch.arange(len(seq_ids), dtype=torch.int32), block_tables=enc,
+        compressed=wl.compressed[seq_ids].cpu(),
+        targets=torch.tensor([[remap[int(p)] for p in row] for row in targets], dtype=torch.int32),
+        pages=used)
