@@ -164,6 +164,30 @@ int zp_compress_score(void* score_cache, const uint8_t* flag, const int32_t* blo
                       int64_t c_stride_layer, int64_t c_stride_page, int64_t c_stride_slot,
                       int64_t c_stride_head, int32_t dtype, void* stream);
 
+/* ---- decode-step neighbours of the compression path (the callers either side of it) ---- */
+
+/* store_kvcache(key, value, k_cache, v_cache, slot_mapping)
+ * zipage/layers/attention.py:12-50 (kernel :12-30): token i of key/value (row_elems = Hkv*D
+ * elements, row stride key_stride/value_stride elements) is copied to slot slot_mapping[i] of
+ * the flat caches (num_slots x row_elems); a slot of -1 skips the token. */
+int zp_store_kvcache(const void* key, const void* value, void* k_cache, void* v_cache,
+                     const int32_t* slot_mapping, int32_t n, int32_t row_elems,
+                     int64_t key_stride, int64_t value_stride, int64_t num_slots,
+                     int32_t dtype, void* stream);
+
+/* Single-query attention over a paged cache, the decode branch of Attention.forward:
+ * zipage/layers/attention.py:95-103 (flash_attn_with_kvcache(q.unsqueeze(1), k_cache, v_cache,
+ * cache_seqlens=context_lens, block_table=block_tables, softmax_scale, causal=True)).
+ * q, out: (B, Hq, D); caches (num_pages, BS, Hkv, D) of one layer with page strides in
+ * elements; block_tables (B, NB) plain page ids (-1 pad); context_lens (B,) tokens attended.
+ * 16-bit caches, D <= 128, GQA group in {1,2,4,8}. */
+int zp_paged_decode_attention(const void* q, const void* k_cache, const void* v_cache,
+                              const int32_t* block_tables, const int32_t* context_lens,
+                              void* out, int32_t B, int32_t Hq, int32_t Hkv, int32_t D,
+                              int32_t BS, int32_t NB, int32_t num_pages,
+                              int64_t k_stride_page, int64_t v_stride_page,
+                              float softmax_scale, int32_t dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

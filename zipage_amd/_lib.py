@@ -41,6 +41,9 @@ SIGNATURES = {
                        i64, i64, i64, i64, i64, i64, i64, i64, i32, ptr],
     "zp_compress_score": [ptr, ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32, i64, i64, i64,
                           i64, i32, ptr],
+    "zp_store_kvcache": [ptr, ptr, ptr, ptr, ptr, i32, i32, i64, i64, i64, i32, ptr],
+    "zp_paged_decode_attention": [ptr, ptr, ptr, ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32,
+                                  i64, i64, f32, i32, ptr],
 }
 I64_RETURNING = {
     "zp_attention_score_workspace": [i32, i32, i32, i32, i32, i32, i32],
