@@ -1,0 +1,156 @@
+"""GPU tests of the decode engine around the compression path, on a tiny random model."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _tiny():
+    from zipage_amd.engine import Qwen3Shape
+    return Qwen3Shape(layers=2, hidden=256, heads=4, kv_heads=2, head_dim=64, intermediate=512,
+                      vocab=503, max_position=2048)
+
+
+def _cfg(**kw):
+    from zipage_amd.compress import CompressConfig
+    from zipage_amd.engine import EngineConfig
+    # the scorer needs 256-token pages for 16-bit caches, so the budget is kept to 2 pages
+    base = dict(shape=_tiny(), max_concurrency=8, num_kvcache_blocks=40, kvcache_block_size=256,
+                max_cache_blocks_per_seq=2, query_cache_len=16, layer_stride=2, seed=5,
+                max_model_len=2048, compress=CompressConfig(enable_pooling=True, pooling_size=3))
+    base.update(kw)
+    return EngineConfig(**base)
+
+
+def _prompts(n, lens, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randint(0, 503, (lens[i % len(lens)],), generator=g).tolist() for i in range(n)]
+
+
+def test_paged_decode_equals_dense_recompute(dev):
+    """Prefill a prefix through the paged caches, decode the rest token by token, and compare
+    every decode step's hidden state with one dense causal pass over the whole sequence.
+    Tolerance: hidden states are RMS-normalised (|x| ~ 1) and pass through 2 bf16 layers; 6e-2
+    absolute covers the bf16 rounding of activations (2^-8 relative per op)."""
+    from zipage_amd.engine import Qwen3, StepContext
+    s = _tiny()
+    BS, pages = 16, 24
+    model = Qwen3(s, dev, seed=11, init_std=0.05)
+    kv = torch.zeros(2, s.layers, pages, BS, s.kv_heads, s.head_dim, device=dev, dtype=torch.bfloat16)
+    qc = torch.zeros(s.layers, 2, 4, s.heads, s.head_dim, device=dev, dtype=torch.bfloat16)
+    n, n0 = 75, 37
+    ids = torch.randint(0, s.vocab, (n,), device=dev)
+    pos = torch.arange(n, device=dev)
+    dense = model.forward(ids, pos, StepContext(True, None, None, None, None, [n], [n])).float()
+    model.attach_caches(kv, qc)
+    table = torch.randperm(pages)[:5].int()
+    slots = (table.long()[:, None] * BS + torch.arange(BS)[None, :]).flatten().int().to(dev)
+    h0 = model.forward(ids[:n0], pos[:n0], StepContext(True, slots[:n0], None, None, None, [n0], [n0]))
+    assert (h0.float() - dense[:n0]).abs().max() < 6e-2
+    tables = table.view(1, 5).to(dev)
+    for t in range(n0, n):
+        ctx = StepContext(False, slots[t:t + 1], None,
+                          torch.tensor([t + 1], device=dev, dtype=torch.int32), tables)
+        h = model.forward(ids[t:t + 1], pos[t:t + 1], ctx)
+        assert (h.float() - dense[t:t + 1]).abs().max() < 6e-2, t
+
+
+def test_cached_prefix_prefill_equals_dense(dev):
+    """Prefill in two parts (the second sees the first through the block table, as a prefix
+    cache hit does) against one dense pass."""
+    from zipage_amd.engine import Qwen3, StepContext
+    s = _tiny()
+    BS, pages = 16, 12
+    model = Qwen3(s, dev, seed=3, init_std=0.05)
+    kv = torch.zeros(2, s.layers, pages, BS, s.kv_heads, s.head_dim, device=dev, dtype=torch.bfloat16)
+    qc = torch.zeros(s.layers, 2, 4, s.heads, s.head_dim, device=dev, dtype=torch.bfloat16)
+    n, n0 = 50, 32
+    ids = torch.randint(0, s.vocab, (n,), device=dev)
+    pos = torch.arange(n, device=dev)
+    dense = model.forward(ids, pos, StepContext(True, None, None, None, None, [n], [n])).float()
+    model.attach_caches(kv, qc)
+    table = torch.tensor([7, 2, 9, 4], dtype=torch.int32)
+    slots = (table.long()[:, None] * BS + torch.arange(BS)[None, :]).flatten().int().to(dev)
+    model.forward(ids[:n0], pos[:n0], StepContext(True, slots[:n0], None, None, None, [n0], [n0]))
+    h = model.forward(ids[n0:], pos[n0:], StepContext(True, slots[n0:n], None, None,
+                                                      table.view(1, 4).to(dev), [n - n0], [n]))
+    assert (h.float() - dense[n0:]).abs().max() < 6e-2
+
+
+def _generate(cfg, prompts, max_tokens):
+    from zipage_amd.engine import SamplingParams, ZipageEngine
+    eng = ZipageEngine(cfg)
+    out = eng.generate(prompts, SamplingParams(max_tokens=max_tokens, ignore_eos=True))
+    return eng, out
+
+
+def test_graph_replay_equals_eager_across_compressions(dev):
+    """The same run with the decode step replayed as a HIP graph and launched eagerly: identical
+    tokens on every step.  Prompts are ragged, so compressions (eager work on the same stream,
+    plus host synchronisations of the pinned ring) fall between replays, and replays cover
+    different padded batch sizes as sequences finish."""
+    prompts = _prompts(5, [90, 300, 470, 640, 1100])
+    e1, a = _generate(_cfg(use_graph=False), prompts, 700)
+    e2, b = _generate(_cfg(use_graph=True), prompts, 700)
+    assert e1.stats["compress_calls"] > 3
+    for x, y in zip(a, b):
+        assert len(x["token_ids"]) == 700
+        assert x["token_ids"] == y["token_ids"]
+        assert x["num_compressions"] == y["num_compressions"] > 0
+
+
+def test_async_compression_bookkeeping(dev):
+    """Side-stream compression: every request still gets all its tokens, each sequence is
+    compressed as often as its length dictates, and all pages and rows come back."""
+    prompts = _prompts(7, [90, 300, 470, 640, 1100, 256, 257], seed=1)
+    cfg = _cfg(enable_async_compress=True, max_compress_blocks=6)
+    eng, out = _generate(cfg, prompts, 600)
+    BS, cap = 256, 3
+    for p, o in zip(prompts, out):
+        assert len(o["token_ids"]) == 600
+        total = len(p) + 600
+        first = max(cap, -(-len(p) // BS)) * BS + 1
+        assert o["num_compressions"] == (0 if total - 1 < first else 1 + (total - 1 - first) // BS)
+    pool = eng.scheduler.pool
+    assert pool.num_free == cfg.num_kvcache_blocks and not pool.refcount.any()
+    assert sorted(eng.scheduler.free_rows) == list(range(cfg.max_concurrency))
+    assert eng.stats["compress_s"] > 0
+
+
+def test_engine_compression_moves_the_right_pages(dev):
+    """Hook the first compression: per layer and head, the rows the target pages hold afterwards
+    are an ordered subset of the rows the sequence's own pages held before (stable gather), and
+    the last `query_cache_len` tokens survive."""
+    from zipage_amd.engine import SamplingParams, ZipageEngine
+    cfg = _cfg(use_graph=False)
+    eng = ZipageEngine(cfg)
+    r = eng.runner
+    seen = {}
+    orig = r.compress
+
+    def hooked(seqs, **kw):
+        if not seen:
+            torch.cuda.synchronize()
+            seen["seqs"] = [(list(s.block_table), list(s.new_block_table)) for s in seqs]
+            seen["k"] = r.kv_cache[0].clone()
+        ev = orig(seqs, **kw)
+        if "after" not in seen:
+            torch.cuda.synchronize()
+            seen["after"] = r.kv_cache[0].clone()
+        return ev
+
+    r.compress = hooked
+    eng.generate(_prompts(3, [700, 750, 200]), SamplingParams(max_tokens=100, ignore_eos=True))
+    assert seen
+    BS, budget, W = 256, 2, 16
+    for table, target in seen["seqs"]:
+        src = seen["k"][:, table].flatten(1, 2)                 # (L, T, Hkv, D)
+        dst = seen["after"][:, target[:budget]].flatten(1, 2)   # (L, budget*BS, Hkv, D)
+        T = src.shape[1]
+        for l in range(src.shape[0]):
+            for h in range(src.shape[2]):
+                eq = (dst[l, :, h, None, :] == src[l, None, :, h, :]).all(-1)   # (kept, T)
+                idx = eq.float().argmax(1)
+                assert eq.any(1).all()
+                assert (idx[1:] > idx[:-1]).all()
+                assert set(range(T - W, T)) <= set(idx.tolist())
