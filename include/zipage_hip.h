@@ -188,6 +188,39 @@ int zp_paged_decode_attention(const void* q, const void* k_cache, const void* v_
                               int64_t k_stride_page, int64_t v_stride_page,
                               float softmax_scale, int32_t dtype, void* stream);
 
+/* ---- fused elementwise pieces of the decoder layer (between the GEMMs and the cache kernels).
+ * The reference takes RMSNorm and SiluAndMul from its nanovllm dependency (imports at
+ * zipage/models/qwen3.py:6-7) and applies per-head q/k norm, rotary embedding, store_kvcache and
+ * store_query_cache as separate modules (zipage/models/qwen3.py:72-88,
+ * zipage/layers/rotary_embedding.py:9-18, zipage/layers/attention.py:69-92). ---- */
+
+/* out = rmsnorm(x [+ residual]) * weight; with a residual pointer the rounded sum is written
+ * back to it (RMSNorm.forward(x, residual) of the dependency).  Strides in elements. */
+int zp_add_rms_norm(const void* x, void* residual, const void* weight, void* out,
+                    int32_t n, int32_t hidden, int64_t x_stride, int64_t r_stride,
+                    int64_t out_stride, float eps, int32_t dtype, void* stream);
+
+/* out = silu(gate_up[:, :I]) * gate_up[:, I:]  (SiluAndMul, zipage/models/qwen3.py:108-111). */
+int zp_silu_and_mul(const void* gate_up, void* out, int32_t n, int32_t intermediate,
+                    int64_t gu_stride, int64_t out_stride, int32_t dtype, void* stream);
+
+/* For every token row of the fused qkv projection: q and k heads are RMS-normalised over the
+ * head (weights q_norm_weight / k_norm_weight), rotated (NeoX halves, cos/sin tables of
+ * (max_position, D/2) fp32 indexed by positions); q goes to q_out (n, Hq, D) and, when
+ * query_triples[i] = (i, query row, ring slot) names the token, into the window ring; k and v go
+ * to slot_mapping[i] of the flat caches (-1 skips); k_out (n, Hkv, D), when given, also receives
+ * the rotated keys (prefill attention reads them).  k_out, query_cache, slot_mapping and
+ * query_triples may be null. */
+int zp_qk_norm_rope_store(const void* qkv, void* q_out, void* k_out, void* k_cache, void* v_cache,
+                          void* query_cache, const void* q_norm_weight,
+                          const void* k_norm_weight, const float* cos, const float* sin,
+                          const int32_t* positions, const int32_t* slot_mapping,
+                          const int32_t* query_triples, int32_t n, int32_t Hq,
+                          int32_t Hkv, int32_t D, int32_t max_position,
+                          int64_t qkv_stride, int64_t num_slots, int32_t max_seqs,
+                          int32_t window, int64_t qc_stride_seq, int64_t qc_stride_slot,
+                          float eps, int32_t dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -44,6 +44,10 @@ SIGNATURES = {
     "zp_store_kvcache": [ptr, ptr, ptr, ptr, ptr, i32, i32, i64, i64, i64, i32, ptr],
     "zp_paged_decode_attention": [ptr, ptr, ptr, ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32,
                                   i64, i64, f32, i32, ptr],
+    "zp_add_rms_norm": [ptr, ptr, ptr, ptr, i32, i32, i64, i64, i64, f32, i32, ptr],
+    "zp_silu_and_mul": [ptr, ptr, i32, i32, i64, i64, i32, ptr],
+    "zp_qk_norm_rope_store": [ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, i32, i32,
+                              i32, i32, i32, i64, i64, i32, i32, i64, i64, f32, i32, ptr],
 }
 I64_RETURNING = {
     "zp_attention_score_workspace": [i32, i32, i32, i32, i32, i32, i32],

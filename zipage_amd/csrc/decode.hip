@@ -31,20 +31,34 @@ __global__ __launch_bounds__(kThreads) void store_kv_kernel(
 }
 
 // ------------------------------------------------------------------ paged decode attention
-template <typename T> __device__ __forceinline__ void unpack8(const u32x4& v, float* o);
-template <> __device__ __forceinline__ void unpack8<BF16>(const u32x4& v, float* o) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    o[2 * i] = __uint_as_float(v[i] << 16);
-    o[2 * i + 1] = __uint_as_float(v[i] & 0xffff0000u);
-  }
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+// acc + a.lo*b.lo + a.hi*b.hi on packed 16-bit pairs, fp32 accumulate (v_dot2_f32_bf16 / _f16)
+template <typename T> __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c);
+template <> __device__ __forceinline__ float dot2<BF16>(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b),
+                                         c, false);
 }
-template <> __device__ __forceinline__ void unpack8<F16>(const u32x4& v, float* o) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    o[2 * i] = f16_bits_to_float((uint16_t)(v[i] & 0xffffu));
-    o[2 * i + 1] = f16_bits_to_float((uint16_t)(v[i] >> 16));
-  }
+template <> __device__ __forceinline__ float dot2<F16>(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), c, false);
+}
+template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi);
+template <> __device__ __forceinline__ uint32_t pack2<BF16>(float lo, float hi) {
+  bf16x2 v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, v);
+}
+template <> __device__ __forceinline__ uint32_t pack2<F16>(float lo, float hi) {
+  f16x2 v = {(_Float16)lo, (_Float16)hi};
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+// Sum over the 8 lanes of a row group, result in all 8 (three DPP stages, no LDS traffic).
+__device__ __forceinline__ float group8_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false));  // row_half_mirror
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+  return v;
 }
 
 struct DecodeArgs {
@@ -59,167 +73,214 @@ struct DecodeArgs {
   float scale;
 };
 
-// One workgroup per (sequence, kv head); G <= 8 query heads share the K/V stream.
-// Pass 1 writes scaled logits (G x T) to LDS, pass 2 the softmax statistics, pass 3 P.V.
+constexpr int kGroups = kThreads / 8;  // token rows in flight per step of the workgroup
+constexpr int kUnroll = 4;             // rows per lane group and loop trip (must be even)
+
+// One workgroup per (sequence, kv head); the G query heads of the group share the K/V stream.
+// Eight lanes own one token row: lane `sub` holds the 16-byte pieces `sub` and `sub + 8` of the
+// head vector, so one load instruction of the wave covers eight rows, each a full 128-byte line.
+//   pass 1: logits = q.k on packed 16-bit pairs, reduced over the 8 lanes, scaled, to LDS (fp32)
+//   pass 2: row maximum, p = exp(logit - max) summed in fp32; p is rounded to the cache dtype and
+//           packed in pairs (token t, token t + 32) over the logit word of t
+//   pass 3: out += p.v with two tokens per dot2 (the pair above), fp32 accumulate; the row
+//           groups are summed at the end and scaled by 1 / sum(p).
 template <typename T, int G>
-__global__ __launch_bounds__(kThreads) void paged_decode_kernel(DecodeArgs p) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(G <= 4 ? 4 : 2, 4))) void paged_decode_kernel(DecodeArgs p) {
   extern __shared__ __align__(16) float lds[];
   __shared__ float red[kWaves * G];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int grp = tid >> 4, sub = tid & 15;     // 16 groups of 16 lanes
+  const int grp = tid >> 3, sub = tid & 7;
   const int h = blockIdx.x % p.Hkv, b = blockIdx.x / p.Hkv;
   int Tn = p.ctx[b];
   Tn = max(0, min(Tn, p.NB * p.BS));
-  const int Tpad = (p.NB * p.BS + 15) & ~15;
+  const int Tpad = (p.NB * p.BS + 63) & ~63;
   float* logit = lds;                            // [G][Tpad]
-  const int dvalid = p.D / 8;                    // 16-byte pieces per head vector (<= 16)
-  const bool on = sub < dvalid;
+  uint32_t* pw = (uint32_t*)lds;                 // packed p pairs over the same words
+  const int pieces = p.D / 8;                    // 16-byte pieces per head vector (<= 16)
+  const bool onA = sub < pieces, onB = sub + 8 < pieces;
   const int64_t row = (int64_t)p.Hkv * p.D * 2;
-  const int64_t hoff = (int64_t)h * p.D * 2 + sub * 16;
-
-  // query pieces of the G heads
-  float qf[G][8];
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    u32x4 raw = {0u, 0u, 0u, 0u};
-    if (on) raw = *(const u32x4*)(p.q + (((int64_t)b * p.Hq + h * G + g) * p.D) * 2 + sub * 16);
-    unpack8<T>(raw, qf[g]);
-#pragma unroll
-    for (int i = 0; i < 8; ++i) qf[g][i] *= p.scale;
-  }
+  const int64_t offA = (int64_t)h * p.D * 2 + (onA ? sub * 16 : 0);
+  const int64_t offB = (int64_t)h * p.D * 2 + (onB ? (sub + 8) * 16 : 0);
   const int32_t* trow = p.table + (int64_t)b * p.NB;
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+
+  auto row_base = [&](const char* cache, int64_t page_stride, int t) -> const char* {
+    const int tc = min(t, Tn - 1);
+    int pid = trow[tc / p.BS];
+    pid = (pid >= 0 && pid < p.num_pages) ? pid : 0;
+    return cache + (int64_t)pid * page_stride * 2 + (int64_t)(tc % p.BS) * row;
+  };
 
   // ---- pass 1: logits
-  for (int t0 = 0; t0 < Tn; t0 += 16 * 4) {
-    u32x4 raw[4];
-    int tt[4];
+  {
+    u32x4 qa[G], qb[G];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int t = t0 + u * 16 + grp;
-      tt[u] = t;
-      const int tc = min(t, Tn - 1);
-      int pid = trow[tc / p.BS];
-      pid = (pid >= 0 && pid < p.num_pages) ? pid : 0;
-      raw[u] = *(const u32x4*)(p.k + (int64_t)pid * p.k_sp * 2 + (int64_t)(tc % p.BS) * row +
-                               (on ? hoff : (int64_t)h * p.D * 2));
+    for (int g = 0; g < G; ++g) {
+      const char* qp = p.q + (((int64_t)b * p.Hq + h * G + g) * p.D) * 2;
+      qa[g] = onA ? *(const u32x4*)(qp + sub * 16) : zero4;
+      qb[g] = onB ? *(const u32x4*)(qp + (sub + 8) * 16) : zero4;
     }
+    // rows of the next trip are requested before the current ones are consumed
+    u32x4 ka[kUnroll], kb[kUnroll], na[kUnroll], nb[kUnroll];
+    auto fetch_k = [&](int t0, u32x4* a, u32x4* bq) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      float kf[8];
-      unpack8<T>(raw[u], kf);
-      float s[G];
+      for (int u = 0; u < kUnroll; ++u) {
+        const char* base = row_base(p.k, p.k_sp, t0 + u * kGroups + grp);
+        a[u] = *(const u32x4*)(base + offA);
+        bq[u] = *(const u32x4*)(base + offB);
+      }
+    };
+    if (Tn > 0) fetch_k(0, ka, kb);
+    for (int t0 = 0; t0 < Tn; t0 += kGroups * kUnroll) {
+      const bool more = t0 + kGroups * kUnroll < Tn;
+      if (more) fetch_k(t0 + kGroups * kUnroll, na, nb);
 #pragma unroll
-      for (int g = 0; g < G; ++g) {
-        float a = 0.f;
-        if (on) {
+      for (int u = 0; u < kUnroll; ++u) {
+        const int t = t0 + u * kGroups + grp;
+        float mine = 0.f;
 #pragma unroll
-          for (int i = 0; i < 8; ++i) a += qf[g][i] * kf[i];
+        for (int g = 0; g < G; ++g) {
+          float a = 0.f;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) a = dot2<T>(ka[u][i], qa[g][i], a);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) a = dot2<T>(kb[u][i], qb[g][i], a);
+          a = group8_sum(a);
+          mine = (sub == g) ? a : mine;
         }
-        s[g] = a;
+        if (sub < G && t < Tn) logit[sub * Tpad + t] = mine * p.scale;
       }
+      if (more) {
 #pragma unroll
-      for (int o = 8; o > 0; o >>= 1) {
-#pragma unroll
-        for (int g = 0; g < G; ++g) s[g] += __shfl_xor(s[g], o, 64);
-      }
-      if (sub == 0 && tt[u] < Tn) {
-#pragma unroll
-        for (int g = 0; g < G; ++g) logit[g * Tpad + tt[u]] = s[g];
+        for (int u = 0; u < kUnroll; ++u) { ka[u] = na[u]; kb[u] = nb[u]; }
       }
     }
   }
   __syncthreads();
-  // ---- pass 2: softmax statistics per head
-  float mx[G], inv[G];
+  // ---- pass 2: softmax statistics per head, p packed in pairs (t, t + 32)
+  float inv[G];
+  {
+    float mx[G];
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float m = -INFINITY;
-    for (int t = tid; t < Tn; t += kThreads) m = fmaxf(m, logit[g * Tpad + t]);
-    m = wave_max(m);
-    if (lane == 0) red[wave * G + g] = m;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float m = red[g];
-    for (int w = 1; w < kWaves; ++w) m = fmaxf(m, red[w * G + g]);
-    mx[g] = m;
-  }
-  __syncthreads();
-#pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float s = 0.f;
-    for (int t = tid; t < Tn; t += kThreads) {
-      const float e = __expf(logit[g * Tpad + t] - mx[g]);
-      logit[g * Tpad + t] = e;
-      s += e;
+    for (int g = 0; g < G; ++g) {
+      float m = -INFINITY;
+      for (int t = tid; t < Tn; t += kThreads) m = fmaxf(m, logit[g * Tpad + t]);
+      m = wave_max(m);
+      if (lane == 0) red[wave * G + g] = m;
     }
-    s = wave_sum(s);
-    if (lane == 0) red[wave * G + g] = s;
-  }
-  __syncthreads();
+    __syncthreads();
 #pragma unroll
-  for (int g = 0; g < G; ++g) {
-    float s = 0.f;
-    for (int w = 0; w < kWaves; ++w) s += red[w * G + g];
-    inv[g] = s > 0.f ? 1.f / s : 0.f;
+    for (int g = 0; g < G; ++g) {
+      float m = red[g];
+      for (int w = 1; w < kWaves; ++w) m = fmaxf(m, red[w * G + g]);
+      mx[g] = m;
+    }
+    __syncthreads();
+    const int npairs = ((Tn + 63) >> 6) * 32;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float s = 0.f;
+      for (int pi = tid; pi < npairs; pi += kThreads) {
+        const int t = (pi >> 5) * 64 + (pi & 31);
+        // each token belongs to exactly one pair, so the packed word can overwrite logit[t]
+        const float e0 = t < Tn ? __expf(logit[g * Tpad + t] - mx[g]) : 0.f;
+        const float e1 = t + 32 < Tn ? __expf(logit[g * Tpad + t + 32] - mx[g]) : 0.f;
+        s += e0 + e1;
+        pw[g * Tpad + t] = pack2<T>(e0, e1);
+      }
+      s = wave_sum(s);
+      if (lane == 0) red[wave * G + g] = s;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      float s = 0.f;
+      for (int w = 0; w < kWaves; ++w) s += red[w * G + g];
+      inv[g] = s > 0.f ? 1.f / s : 0.f;
+    }
   }
-  // ---- pass 3: P.V, each 16-lane group accumulates its tokens
+  // ---- pass 3: P.V, two tokens per dot2.  Sixteen lanes per row here (one 16-byte piece each),
+  // which halves the accumulators a lane carries; a trip covers two 64-token blocks, and row
+  // group `g16` takes the pairs j = g16 and j = g16 + 16 of each.
+  const int g16 = tid >> 4, s16 = tid & 15;
+  const bool onV = s16 < pieces;
+  const int64_t offV = (int64_t)h * p.D * 2 + (onV ? s16 * 16 : 0);
   float acc[G][8];
 #pragma unroll
   for (int g = 0; g < G; ++g)
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
-  for (int t0 = 0; t0 < Tn; t0 += 16 * 4) {
-    u32x4 raw[4];
-    int tt[4];
+  constexpr int kPairs = 4;
+  u32x4 vx[kPairs], vy[kPairs], nx[kPairs], ny[kPairs];
+  auto fetch_v = [&](int t0, u32x4* x, u32x4* y) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int t = t0 + u * 16 + grp;
-      tt[u] = t;
-      const int tc = min(t, Tn - 1);
-      int pid = trow[tc / p.BS];
-      pid = (pid >= 0 && pid < p.num_pages) ? pid : 0;
-      raw[u] = *(const u32x4*)(p.v + (int64_t)pid * p.v_sp * 2 + (int64_t)(tc % p.BS) * row +
-                               (on ? hoff : (int64_t)h * p.D * 2));
+    for (int u = 0; u < kPairs; ++u) {
+      const int t = t0 + (u >> 1) * 64 + (u & 1) * 16 + g16;
+      x[u] = *(const u32x4*)(row_base(p.v, p.v_sp, t) + offV);
+      y[u] = *(const u32x4*)(row_base(p.v, p.v_sp, t + 32) + offV);
     }
+  };
+  if (Tn > 0) fetch_v(0, vx, vy);
+  for (int t0 = 0; t0 < Tn; t0 += 16 * kPairs * 2) {
+    const bool more = t0 + 16 * kPairs * 2 < Tn;
+    if (more) fetch_v(t0 + 16 * kPairs * 2, nx, ny);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      float vf[8];
-      unpack8<T>(raw[u], vf);
-      if (tt[u] < Tn) {
+    for (int u = 0; u < kPairs; ++u) {
+      const int t = t0 + (u >> 1) * 64 + (u & 1) * 16 + g16;  // partner is t + 32
+      if (t < Tn) {
+        uint32_t pp[G];
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
-          const float pw = logit[g * Tpad + tt[u]];
+        for (int g = 0; g < G; ++g) pp[g] = pw[g * Tpad + t];
 #pragma unroll
-          for (int i = 0; i < 8; ++i) acc[g][i] += pw * vf[i];
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t lo = __builtin_amdgcn_perm(vy[u][i], vx[u][i], 0x05040100u);  // (x.lo16, y.lo16)
+          const uint32_t hi = __builtin_amdgcn_perm(vy[u][i], vx[u][i], 0x07060302u);  // (x.hi16, y.hi16)
+#pragma unroll
+          for (int g = 0; g < G; ++g) {
+            acc[g][2 * i] = dot2<T>(lo, pp[g], acc[g][2 * i]);
+            acc[g][2 * i + 1] = dot2<T>(hi, pp[g], acc[g][2 * i + 1]);
+          }
         }
       }
     }
+    if (more) {
+#pragma unroll
+      for (int u = 0; u < kPairs; ++u) { vx[u] = nx[u]; vy[u] = ny[u]; }
+    }
   }
-  __syncthreads();  // logits no longer needed: reuse the LDS for the cross-group reduction
-  float* part = lds;  // [16 groups][G][128]
-  if (on) {
+  // sum the 4 row groups of each wave (lanes with equal piece), then the waves through LDS
+#pragma unroll
+  for (int g = 0; g < G; ++g)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float v = acc[g][i];
+      v += __shfl_xor(v, 16, 64);
+      v += __shfl_xor(v, 32, 64);
+      acc[g][i] = v;
+    }
+  __syncthreads();  // p no longer needed: reuse the LDS
+  float* part = lds;  // [kWaves][G][128]
+  if (lane < 16) {
 #pragma unroll
     for (int g = 0; g < G; ++g)
 #pragma unroll
-      for (int i = 0; i < 8; ++i) part[(grp * G + g) * 128 + sub * 8 + i] = acc[g][i];
+      for (int i = 0; i < 8; ++i) part[(wave * G + g) * 128 + s16 * 8 + i] = acc[g][i];
   }
   __syncthreads();
   for (int e = tid; e < G * p.D; e += kThreads) {
     const int g = e / p.D, d = e - g * p.D;
     float s = 0.f;
 #pragma unroll
-    for (int q = 0; q < 16; ++q) s += part[(q * G + g) * 128 + d];
+    for (int w = 0; w < kWaves; ++w) s += part[(w * G + g) * 128 + d];
     Elem<T>::st(p.out, ((int64_t)b * p.Hq + h * G + g) * p.D + d, s * inv[g]);
   }
 }
 
 template <typename T, int G>
 int launch_decode(const DecodeArgs& a, hipStream_t st) {
-  const int Tpad = (a.NB * a.BS + 15) & ~15;
+  const int Tpad = (a.NB * a.BS + 63) & ~63;
   size_t smem = sizeof(float) * (size_t)G * Tpad;
-  const size_t part = sizeof(float) * 16 * G * 128;
+  const size_t part = sizeof(float) * kWaves * G * 128;
   if (part > smem) smem = part;
   if (smem > 150 * 1024) {
     zp_set_error("paged_decode_attention: %d cached tokens x %d heads exceed LDS", a.NB * a.BS, G);

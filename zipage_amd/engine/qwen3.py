@@ -1,9 +1,10 @@
 """Random-initialised Qwen3 decoder (zipage/models/qwen3.py) wired to the paged caches.
 
-Only what the decode benchmark needs: bf16 weights drawn on the device, fused qkv and gate/up
-projections through torch's GEMMs, per-head q/k RMSNorm, NeoX rotary embedding, and the three
-cache-side kernels of this package inside every attention layer (store_kvcache, store_query_cache,
-paged decode attention).  Prefill attention is torch's scaled_dot_product_attention.
+Only what the decode benchmark needs: bf16 weights drawn on the device and the fused qkv and
+gate/up projections through torch's GEMMs; everything between the GEMMs is this package's HIP
+kernels (residual add + RMSNorm, per-head q/k norm + rotary embedding + K/V scatter + window-query
+capture, paged decode attention, SiLU gate).  Prefill attention is torch's
+scaled_dot_product_attention.
 """
 from __future__ import annotations
 
@@ -13,7 +14,7 @@ import torch
 import torch.nn.functional as F
 
 from zipage_amd.kernel import store_query_cache
-from zipage_amd.layers import paged_decode_attention, store_kvcache
+from zipage_amd.layers import paged_decode_attention, qk_norm_rope_store, rms_norm, silu_and_mul
 
 
 @dataclass(frozen=True)
@@ -45,10 +46,6 @@ class StepContext:
     block_tables: torch.Tensor | None = None        # (B, NB) int32, decode / cached prefill
     seq_lens_q: list[int] | None = None             # prefill: new tokens per sequence
     seq_lens_k: list[int] | None = None             # prefill: total tokens per sequence
-
-
-def _rms(x: torch.Tensor, w: torch.Tensor, eps: float) -> torch.Tensor:
-    return F.rms_norm(x, (x.shape[-1],), w, eps)
 
 
 class Qwen3:
@@ -85,11 +82,6 @@ class Qwen3:
         self.k_cache, self.v_cache, self.q_cache = kv_cache[0], kv_cache[1], query_cache
 
     # ------------------------------------------------------------------ pieces
-    def _rope(self, x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
-        """zipage/layers/rotary_embedding.py:9-18: NeoX halves, computed in fp32."""
-        x1, x2 = x.float().chunk(2, dim=-1)
-        return torch.cat((x1 * cos - x2 * sin, x2 * cos + x1 * sin), dim=-1).to(x.dtype)
-
     def _prefill_attention(self, li, q, k, v, ctx: StepContext) -> torch.Tensor:
         s = self.shape
         lens_q, lens_k = ctx.seq_lens_q, ctx.seq_lens_k
@@ -120,46 +112,51 @@ class Qwen3:
             off += nq
         return out.view(-1, s.heads * s.head_dim)
 
-    def _attention(self, li, p, x, cos, sin, ctx: StepContext) -> torch.Tensor:
+    def _attention(self, li, p, x, pos32, ctx: StepContext) -> torch.Tensor:
         """zipage/models/qwen3.py:72-88 + zipage/layers/attention.py:69-104."""
         s = self.shape
         N = x.shape[0]
         qkv = F.linear(x, p["wqkv"])
         q_sz, kv_sz = s.heads * s.head_dim, s.kv_heads * s.head_dim
-        q = qkv[:, :q_sz].view(N, s.heads, s.head_dim)
-        k = qkv[:, q_sz:q_sz + kv_sz].view(N, s.kv_heads, s.head_dim)
-        v = qkv[:, q_sz + kv_sz:].view(N, s.kv_heads, s.head_dim)
-        q = self._rope(_rms(q, p["qn"], s.eps), cos, sin)
-        k = self._rope(_rms(k, p["kn"], s.eps), cos, sin)
-        if self.k_cache is not None and self.k_cache.numel() and ctx.slot_mapping is not None:
-            store_kvcache(k, v, self.k_cache[li], self.v_cache[li], ctx.slot_mapping)
-        if ctx.query_slot_mapping is not None:
-            store_query_cache(q, self.q_cache[li], ctx.query_slot_mapping)
+        cached = self.k_cache is not None and self.k_cache.numel() > 0 and ctx.slot_mapping is not None
+        kc = self.k_cache[li] if cached else None
+        vc = self.v_cache[li] if cached else None
         if ctx.is_prefill:
+            q, k = qk_norm_rope_store(qkv, pos32, self.cos, self.sin, p["qn"], p["kn"], s.heads,
+                                      s.kv_heads, s.head_dim, s.eps, kc, vc,
+                                      ctx.slot_mapping if cached else None, return_k=True)
+            if ctx.query_slot_mapping is not None:
+                store_query_cache(q, self.q_cache[li], ctx.query_slot_mapping)
+            v = qkv[:, q_sz + kv_sz:].view(N, s.kv_heads, s.head_dim)
             o = self._prefill_attention(li, q, k, v, ctx)
         else:
-            o = paged_decode_attention(q, self.k_cache[li], self.v_cache[li], ctx.context_lens,
-                                       ctx.block_tables, self.scale).view(N, q_sz)
+            q = qk_norm_rope_store(qkv, pos32, self.cos, self.sin, p["qn"], p["kn"], s.heads,
+                                   s.kv_heads, s.head_dim, s.eps, kc, vc, ctx.slot_mapping,
+                                   self.q_cache[li] if ctx.query_slot_mapping is not None else None,
+                                   ctx.query_slot_mapping)
+            o = paged_decode_attention(q, kc, vc, ctx.context_lens, ctx.block_tables,
+                                       self.scale).view(N, q_sz)
         return F.linear(o, p["wo"])
-
-    def _mlp(self, p, x) -> torch.Tensor:
-        gu = F.linear(x, p["wgu"])
-        g, u = gu.chunk(2, dim=-1)
-        return F.linear(F.silu(g) * u, p["wd"])
 
     # ------------------------------------------------------------------ forward
     @torch.inference_mode()
     def forward(self, input_ids: torch.Tensor, positions: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        """Hidden states (N, hidden) after the final norm (zipage/models/qwen3.py:169-181)."""
+        """Hidden states (N, hidden) after the final norm (zipage/models/qwen3.py:169-181).  In a
+        decode step `ctx.query_slot_mapping` holds one triple per token (row -1 = none)."""
         s = self.shape
-        cos = self.cos[positions].unsqueeze(1)      # (N, 1, D/2)
-        sin = self.sin[positions].unsqueeze(1)
-        resid = F.embedding(input_ids, self.embed)
+        pos32 = positions.to(torch.int32)
+        hidden = F.embedding(input_ids, self.embed)
+        resid = None
         for li, p in enumerate(self.layers):
-            h = self._attention(li, p, _rms(resid, p["ln1"], s.eps), cos, sin, ctx)
-            resid = resid + h
-            resid = resid + self._mlp(p, _rms(resid, p["ln2"], s.eps))
-        return _rms(resid, self.final_norm, s.eps)
+            if resid is None:
+                resid, h = hidden, rms_norm(hidden, p["ln1"], s.eps)
+            else:
+                h, resid = rms_norm(hidden, p["ln1"], s.eps, resid)
+            hidden = self._attention(li, p, h, pos32, ctx)
+            h, resid = rms_norm(hidden, p["ln2"], s.eps, resid)
+            hidden = F.linear(silu_and_mul(F.linear(h, p["wgu"])), p["wd"])
+        h, _ = rms_norm(hidden, self.final_norm, s.eps, resid)
+        return h
 
     @torch.inference_mode()
     def compute_logits(self, hidden: torch.Tensor) -> torch.Tensor:
