@@ -6,7 +6,12 @@ top-2048 per kv head -> in-place compaction to 8 pages) over one batch of synthe
 sequences at Qwen3-8B attention shape (32 q heads, 8 kv heads, head_dim 128, bf16, page 256,
 window 32), one layer, inputs resident in HBM.  Prints ONE JSON line.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--no-cpu-baseline]
+After it, unless --no-e2e, the same process runs BASELINE's end-to-end case (random-init
+Qwen3-8B, 256 requests x 512-token prompts x 4096 greedy tokens, budget 8 pages) through the
+decode engine and adds decode tokens/s and the compression share as `end_to_end`.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--no-cpu-baseline] [--no-e2e]
+  python bench.py --config 5 [--requests R] [--prompt P] [--out-tokens T] [--sync-compress]
 """
 from __future__ import annotations
 
@@ -57,17 +62,92 @@ def cpu_baseline(wl, cfg, sample_seqs, budget_s=30.0):
                       f"after 1 warm-up ({med * 1e3:.0f} ms per run)"}
 
 
+def end_to_end(requests=256, prompt=512, out_tokens=4096, async_compress=True, ragged=False):
+    """BASELINE configs[4]: offline decode of a random-init Qwen3-8B with the KV budget on.
+    Returns decode tokens/s (decode steps only, first decode step to the last, device-complete),
+    the share of that time the compression kernels were running, and the bandwidth of the
+    decode-attention kernel at the steady-state shape."""
+    import torch
+    from zipage_amd.compress import CompressConfig
+    from zipage_amd.engine import QWEN3_8B, EngineConfig, SamplingParams, ZipageEngine
+    from zipage_amd.layers import paged_decode_attention
+
+    cfg = EngineConfig(shape=QWEN3_8B, max_concurrency=requests,
+                       num_kvcache_blocks=requests * 9 + 64, query_cache_len=16,
+                       max_model_len=prompt + out_tokens + 1, enable_async_compress=async_compress,
+                       max_compress_blocks=requests * 16,
+                       compress=CompressConfig(enable_pooling=True, pooling_size=5))
+    eng = ZipageEngine(cfg)
+    g = torch.Generator().manual_seed(0)
+    if ragged:
+        lens = torch.randint(prompt // 2, prompt + prompt // 2 + 1, (requests,), generator=g).tolist()
+    else:
+        lens = [prompt] * requests
+    prompts = [torch.randint(0, QWEN3_8B.vocab, (n,), generator=g).tolist() for n in lens]
+    outs = eng.generate(prompts, SamplingParams(max_tokens=out_tokens, ignore_eos=True))
+    st = eng.stats
+    assert all(len(o["token_ids"]) == out_tokens for o in outs)
+    # decode attention alone, at the steady-state shape of this run (8 full pages + half a page)
+    r = eng.runner
+    B, BS = requests, cfg.kvcache_block_size
+    ctx_len = min(8 * BS + BS // 2, prompt + out_tokens)
+    tables = torch.arange(B * 9, device=r.device, dtype=torch.int32).view(B, 9)
+    ctx = torch.full((B,), ctx_len, device=r.device, dtype=torch.int32)
+    q = torch.randn(B, QWEN3_8B.heads, QWEN3_8B.head_dim, device=r.device).to(torch.bfloat16)
+    kc, vc = r.kv_cache[0, 0], r.kv_cache[1, 0]
+    for _ in range(3):
+        paged_decode_attention(q, kc, vc, ctx, tables, 128 ** -0.5)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(20):
+        paged_decode_attention(q, kc, vc, ctx, tables, 128 ** -0.5)
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) / 20 * 1e3
+    alg = B * ctx_len * QWEN3_8B.kv_heads * QWEN3_8B.head_dim * 2 * 2   # K and V rows, read once
+    out = {
+        "workload": (f"configs[4]: random-init Qwen3-8B bf16, {requests} requests, "
+                     f"{'ragged ' if ragged else ''}{prompt}-token prompts, {out_tokens} greedy tokens "
+                     "each, budget 8 pages x 256 tokens, window 16, max-pool 5, compression "
+                     + ("on a side stream" if async_compress else "in line with the decode steps")),
+        "decode_tok_per_s": round(st["decode_tokens"] / st["decode_s"], 1),
+        "ms_per_decode_step": round(st["decode_s"] / st["decode_steps"] * 1e3, 3),
+        "decode_steps": st["decode_steps"],
+        "prefill_tok_per_s": round(st["prefill_tokens"] / st["prefill_s"], 1),
+        "compress_calls": st["compress_calls"], "sequences_compressed": st["compress_seqs"],
+        "compress_share_of_decode_time": round(st["compress_s"] / st["decode_s"], 5),
+        "decode_attention": {"bound": "hbm", "kernel": "paged_decode_kernel",
+                             "avg_launch_us": round(us, 1), "algorithmic_bytes": alg,
+                             "achieved": round(alg / us / 1e3, 1), "peak": HBM_PEAK_GBS,
+                             "unit": "GB/s", "frac": round(alg / us / 1e3 / HBM_PEAK_GBS, 4)},
+    }
+    del eng
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--batch", type=int, default=None)
-    ap.add_argument("--config", type=int, default=2, choices=[2, 4],
+    ap.add_argument("--config", type=int, default=2, choices=[2, 4, 5],
                     help="BASELINE config (1-based as in SURVEY): 2 = 64 ragged sequences, one "
                          "layer (default, the headline line); 4 = 256 sequences with shared "
                          "prefixes and copy-on-write targets, 36 layers run one layer at a time "
-                         "over one page pool")
+                         "over one page pool; 5 = the end-to-end decode case alone")
+    ap.add_argument("--no-e2e", action="store_true",
+                    help="skip the end-to-end decode leg that follows the default run")
+    ap.add_argument("--requests", type=int, default=256)
+    ap.add_argument("--prompt", type=int, default=512)
+    ap.add_argument("--out-tokens", type=int, default=4096)
+    ap.add_argument("--sync-compress", action="store_true",
+                    help="end-to-end leg: compress in line with the decode steps instead of on "
+                         "the side stream")
+    ap.add_argument("--ragged-prompts", action="store_true",
+                    help="end-to-end leg: prompt lengths uniform in [P/2, 3P/2] so sequences reach "
+                         "their budget on different steps")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", type=int, default=64)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -91,6 +171,17 @@ def main():
 
     _lib.load()  # fail loudly if the HIP library is missing
     torch.cuda.set_device(0)
+    if args.config == 5:
+        e2e = end_to_end(args.requests, args.prompt, args.out_tokens, not args.sync_compress,
+                         args.ragged_prompts)
+        print(json.dumps({
+            "metric": "decode tokens/sec", "value": e2e["decode_tok_per_s"], "unit": "tokens/s",
+            "n_gpus": 1, "steps": e2e["decode_steps"], "warmup": 0,
+            "ms_per_step": e2e["ms_per_decode_step"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": e2e["workload"]}, "roofline": e2e["decode_attention"],
+            "cpu_baseline": None, "end_to_end": e2e}))
+        return
     if args.config == 2:
         batch, layers = args.batch or 64, 1
         wl = ragged_batch(batch, L=1, pool_pages=20000, budget=8, W=32, seed=1,
@@ -162,6 +253,11 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl, cfg, args.cpu_sample)
+    if not args.no_e2e and args.config == 2 and args.batch is None:
+        del wl
+        torch.cuda.empty_cache()
+        out["end_to_end"] = end_to_end(args.requests, args.prompt, args.out_tokens,
+                                       not args.sync_compress, args.ragged_prompts)
     print(json.dumps(out))
 
 

@@ -23,7 +23,7 @@ class EngineConfig:
     query_cache_len: int = 16
     layer_stride: int = 8               # layers per compression launch (model_runner.py:466)
     enable_async_compress: bool = False
-    max_compress_blocks: int = 600      # pages one asynchronous compression may cover
+    max_compress_blocks: int = 4096     # pages one asynchronous compression may cover
     enable_prefix_cache: bool = False
     use_graph: bool = True              # replay the decode step as a HIP graph
     seed: int = 0
