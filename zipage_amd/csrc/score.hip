@@ -36,6 +36,9 @@ constexpr int kRowWaves = 4;   // most waves along the query-row axis; the other
                                // Fewer row blocks (small window x group) use 2 or 1 row waves so
                                // that no wave idles: ScoreArgs::RW.
 constexpr int kDmax = 128;
+#ifndef ZP_SCORE_ZIGZAG
+#define ZP_SCORE_ZIGZAG 1
+#endif
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
@@ -271,15 +274,19 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? 2 : 1)) v
       float run[16];
 #pragma unroll
       for (int r = 0; r < 16; ++r) run[r] = PASS == 0 ? -INFINITY : 0.f;
+      // The middle sweep walks the tiles backwards: it starts on the tiles the first sweep read
+      // last (still in L2) and ends on those the third sweep reads first.
+      auto order = [&](int i) { return (ZP_SCORE_ZIGZAG && PASS == 1) ? ntiles - 1 - i : i; };
       if (ntiles > 0) {
-        issue_loads(0);
+        issue_loads(order(0));
         commit_loads(kbuf0);
       }
       __syncthreads();
-      for (int tile = 0; tile < ntiles; ++tile) {
-        char* cur = (tile & 1) ? kbuf1 : kbuf0;
-        char* nxt = (tile & 1) ? kbuf0 : kbuf1;
-        if (tile + 1 < ntiles) issue_loads(tile + 1);
+      for (int it = 0; it < ntiles; ++it) {
+        const int tile = order(it);
+        char* cur = (it & 1) ? kbuf1 : kbuf0;
+        char* nxt = (it & 1) ? kbuf0 : kbuf1;
+        if (it + 1 < ntiles) issue_loads(order(it + 1));
         const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
         const int j = vslot[vp] & 0xffff;
         const bool last = (vslot[vp] >> 30) & 1;
@@ -403,7 +410,7 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? 2 : 1)) v
           for (int sti = 0; sti < NSUB; ++sti)
             if (half == 0) part[((tile & 1) * kRowWaves + rbw) * TN + (tg * NSUB + sti) * 32 + col] = 0.f;
         }
-        if (tile + 1 < ntiles) commit_loads(nxt);
+        if (it + 1 < ntiles) commit_loads(nxt);
         __syncthreads();
         // the window partials of this tile are complete: combine the waves' shares while the
         // next tile is being computed (the buffer is rewritten two tiles later)
