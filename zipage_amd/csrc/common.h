@@ -88,20 +88,62 @@ __device__ __forceinline__ bool page_is_last(int code) { return code < -1; }
 __device__ __forceinline__ int page_id(int code) { return code < -1 ? -code - 2 : code; }
 
 // ---------------------------------------------------------------- wave helpers
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+// Cross-lane exchanges without the LDS crossbar: DPP rotations inside a row of 16 lanes, and the
+// gfx950 lane-swap instructions for the two wider steps.  A ds_bpermute round trip costs a
+// hundred-odd cycles of latency; these are ordinary VALU instructions.
+template <int N> __device__ __forceinline__ int dpp_row_ror(int x) {
+  return __builtin_amdgcn_update_dpp(0, x, 0x120 + N, 0xf, 0xf, false);  // lane i <- lane (i+N)%16 of its row
+}
+template <int N> __device__ __forceinline__ float dpp_row_ror(float x) {
+  return __builtin_bit_cast(float, dpp_row_ror<N>(__builtin_bit_cast(int, x)));
+}
+// value of lane ^ 16 (v_permlane16_swap: odd rows of one operand <-> even rows of the other)
+__device__ __forceinline__ int lane_xor16(int x) {
+  const auto r = __builtin_amdgcn_permlane16_swap((unsigned)x, (unsigned)x, false, false);
+  return (int)((threadIdx.x & 16) ? r[0] : r[1]);
+}
+__device__ __forceinline__ float lane_xor16(float x) {
+  return __builtin_bit_cast(float, lane_xor16(__builtin_bit_cast(int, x)));
+}
+// value of lane ^ 32 (v_permlane32_swap: upper half of one operand <-> lower half of the other)
+__device__ __forceinline__ int lane_xor32(int x) {
+  const auto r = __builtin_amdgcn_permlane32_swap((unsigned)x, (unsigned)x, false, false);
+  return (int)((threadIdx.x & 32) ? r[0] : r[1]);
+}
+__device__ __forceinline__ float lane_xor32(float x) {
+  return __builtin_bit_cast(float, lane_xor32(__builtin_bit_cast(int, x)));
+}
+// all-reduce over the 16 lanes of a row (every lane ends with the result)
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_row_ror<8>(v);
+  v += dpp_row_ror<4>(v);
+  v += dpp_row_ror<2>(v);
+  v += dpp_row_ror<1>(v);
   return v;
 }
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+__device__ __forceinline__ int row16_sum(int v) {
+  v += dpp_row_ror<8>(v);
+  v += dpp_row_ror<4>(v);
+  v += dpp_row_ror<2>(v);
+  v += dpp_row_ror<1>(v);
   return v;
 }
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_row_ror<8>(v));
+  v = fmaxf(v, dpp_row_ror<4>(v));
+  v = fmaxf(v, dpp_row_ror<2>(v));
+  v = fmaxf(v, dpp_row_ror<1>(v));
+  return v;
+}
+// all-reduce over 32 lanes (each half of the wave separately) and over the whole wave
+__device__ __forceinline__ float half_sum(float v) { v = row16_sum(v); return v + lane_xor16(v); }
+__device__ __forceinline__ float half_max(float v) { v = row16_max(v); return fmaxf(v, lane_xor16(v)); }
+__device__ __forceinline__ float wave_max(float v) { v = half_max(v); return fmaxf(v, lane_xor32(v)); }
+__device__ __forceinline__ float wave_sum(float v) { v = half_sum(v); return v + lane_xor32(v); }
 __device__ __forceinline__ int wave_sum_i(int v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
+  v = row16_sum(v);
+  v += lane_xor16(v);
+  return v + lane_xor32(v);
 }
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }

@@ -257,8 +257,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(G <= 4
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       float v = acc[g][i];
-      v += __shfl_xor(v, 16, 64);
-      v += __shfl_xor(v, 32, 64);
+      v += lane_xor16(v);
+      v += lane_xor32(v);
       acc[g][i] = v;
     }
   __syncthreads();  // p no longer needed: reuse the LDS

@@ -18,6 +18,29 @@
 
 namespace {
 
+// Sum over the PIECES (16 or 32) consecutive lanes that hold one key row.
+template <int PIECES> __device__ __forceinline__ float pieces_sum(float v) {
+  static_assert(PIECES == 16 || PIECES == 32, "a key row spans 16 or 32 lanes");
+  v = row16_sum(v);
+  if (PIECES == 32) v += lane_xor16(v);
+  return v;
+}
+// Over the 32 lanes of a wave half: the entry with the largest column index (and its value).
+__device__ __forceinline__ void last_claim_reduce(int& c, float& v) {
+#define ZP_CLAIM_STEP(OC, OV)              \
+  do {                                     \
+    const int oc_ = (OC);                  \
+    const float ov_ = (OV);                \
+    if (oc_ > c) { c = oc_; v = ov_; }     \
+  } while (0)
+  ZP_CLAIM_STEP(dpp_row_ror<8>(c), dpp_row_ror<8>(v));
+  ZP_CLAIM_STEP(dpp_row_ror<4>(c), dpp_row_ror<4>(v));
+  ZP_CLAIM_STEP(dpp_row_ror<2>(c), dpp_row_ror<2>(v));
+  ZP_CLAIM_STEP(dpp_row_ror<1>(c), dpp_row_ror<1>(v));
+  ZP_CLAIM_STEP(lane_xor16(c), lane_xor16(v));
+#undef ZP_CLAIM_STEP
+}
+
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
 constexpr int kDmax = 128;
@@ -152,8 +175,7 @@ __global__ __launch_bounds__(kThreads) void gram_kernel(GramArgs p) {
       float ss = 0.f;
 #pragma unroll
       for (int q = 0; q < NE; ++q) ss += e[q] * e[q];
-#pragma unroll
-      for (int o = PIECES >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      ss = pieces_sum<PIECES>(ss);
       const float n = fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
       if (st_piece < dpieces) {
         float* d = buf + row * ROWF + st_piece * NE;
@@ -234,13 +256,8 @@ __global__ __launch_bounds__(kThreads) void gram_kernel(GramArgs p) {
       float s = rsum[r];
       int c = ccol[r];
       float v = cval[r];
-#pragma unroll
-      for (int o = 16; o > 0; o >>= 1) {
-        s += __shfl_xor(s, o, 64);
-        const int oc = __shfl_xor(c, o, 64);
-        const float ov = __shfl_xor(v, o, 64);
-        if (oc > c) { c = oc; v = ov; }
-      }
+      s = half_sum(s);
+      last_claim_reduce(c, v);
       if (active && col == 0) {
         const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
         if (RAW) {
@@ -367,8 +384,7 @@ __global__ __launch_bounds__(kThreads, 2) void gram_split_kernel(GramArgs p) {
 #pragma unroll
         for (int q = 0; q < 8; ++q) ss += e[q] * e[q];
       }
-#pragma unroll
-      for (int o = PIECES >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      ss = pieces_sum<PIECES>(ss);
       const float n = fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
       if (st_piece < dpieces) {
 #pragma unroll
@@ -402,7 +418,7 @@ __global__ __launch_bounds__(kThreads, 2) void gram_split_kernel(GramArgs p) {
 #pragma unroll
         for (int q = 0; q < 8; ++q) ss += x[s][q] * x[s][q];
       }
-      ss += __shfl_xor(ss, 32, 64);  // the other half of the row
+      ss += lane_xor32(ss);  // the other half of the row
       const float n = fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
 #pragma unroll
       for (int s = 0; s < KSB; ++s) {
@@ -468,13 +484,8 @@ __global__ __launch_bounds__(kThreads, 2) void gram_split_kernel(GramArgs p) {
       float s = rsum[r];
       int c = ccol[r];
       float v = cval[r];
-#pragma unroll
-      for (int o = 16; o > 0; o >>= 1) {
-        s += __shfl_xor(s, o, 64);
-        const int oc = __shfl_xor(c, o, 64);
-        const float ov = __shfl_xor(v, o, 64);
-        if (oc > c) { c = oc; v = ov; }
-      }
+      s = half_sum(s);
+      last_claim_reduce(c, v);
       if (active && col == 0) {
         const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
         if (RAW) {
@@ -568,8 +579,7 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
 #pragma unroll
         for (int q = 0; q < 8; ++q) ss += e[q] * e[q];
       }
-#pragma unroll
-      for (int o = PIECES >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      ss = pieces_sum<PIECES>(ss);
       const float rn = 1.f / fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
       bf16x8_t hi, lo;
 #pragma unroll
@@ -635,13 +645,8 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
       float s = rsum[r];
       int c = ccol[r];
       float v = cval[r];
-#pragma unroll
-      for (int o = 16; o > 0; o >>= 1) {
-        s += __shfl_xor(s, o, 64);
-        const int oc = __shfl_xor(c, o, 64);
-        const float ov = __shfl_xor(v, o, 64);
-        if (oc > c) { c = oc; v = ov; }
-      }
+      s = half_sum(s);
+      last_claim_reduce(c, v);
       if (col == 0) {
         const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
         l_sum[rslot] = s;

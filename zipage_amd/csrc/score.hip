@@ -369,7 +369,7 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? 2 : 1)) v
                     q4[q] = fmaxf(fmaxf(pv[4 * q], pv[4 * q + 1]), fmaxf(pv[4 * q + 2], pv[4 * q + 3]));
                   if (Gp >= 8) {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) q4[q] = fmaxf(q4[q], __shfl_xor(q4[q], 32, 64));
+                    for (int q = 0; q < 4; ++q) q4[q] = fmaxf(q4[q], lane_xor32(q4[q]));
                   }
                   if (Gp >= 16) {
                     q4[0] = fmaxf(q4[0], q4[1]);
@@ -398,7 +398,7 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? 2 : 1)) v
                   }
                 }
                 if (Gp < 8) {  // the two lane halves hold different windows
-                  const float o = __shfl_xor(red, 32, 64);
+                  const float o = lane_xor32(red);
                   red = p.reduce_max ? fmaxf(red, o) : red + o;
                 }
                 if (half == 0) part[((tile & 1) * kRowWaves + rbw) * TN + st * 32 + col] = red;
@@ -421,12 +421,7 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? 2 : 1)) v
       if constexpr (PASS < 2) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          float v = run[r];
-#pragma unroll
-          for (int o = 16; o > 0; o >>= 1) {
-            const float t = __shfl_xor(v, o, 64);
-            v = PASS == 0 ? fmaxf(v, t) : v + t;
-          }
+          const float v = PASS == 0 ? half_max(run[r]) : half_sum(run[r]);
           run[r] = v;
           if (col == 0) stat[wave * 32 + (r >> 2) * 8 + half * 4 + (r & 3)] = v;
         }
