@@ -154,3 +154,62 @@ def test_engine_compression_moves_the_right_pages(dev):
                 assert eq.any(1).all()
                 assert (idx[1:] > idx[:-1]).all()
                 assert set(range(T - W, T)) <= set(idx.tolist())
+
+
+def test_eos_stops_a_request_and_frees_its_pages(dev):
+    """A request without ignore_eos ends at the first EOS it samples (token values travel to the
+    host every step in that case); the others run to max_tokens."""
+    from zipage_amd.engine import SamplingParams, ZipageEngine
+    prompts = _prompts(3, [40, 300, 90], seed=4)
+    ref, out = _generate(_cfg(use_graph=False), prompts, 60)
+    eos = out[0]["token_ids"][20]
+    first = out[0]["token_ids"].index(eos)
+    cfg = _cfg(use_graph=False, eos=eos)
+    eng = ZipageEngine(cfg)
+    params = [SamplingParams(max_tokens=60, ignore_eos=False)] + [SamplingParams(max_tokens=60, ignore_eos=True)] * 2
+    got = eng.generate(prompts, params)
+    assert got[0]["token_ids"] == out[0]["token_ids"][:first + 1]
+    assert got[1]["token_ids"] == out[1]["token_ids"] and got[2]["token_ids"] == out[2]["token_ids"]
+    assert eng.scheduler.pool.num_free == cfg.num_kvcache_blocks
+
+
+def test_temperature_sampling_runs_eagerly(dev):
+    from zipage_amd.engine import SamplingParams, ZipageEngine
+    cfg = _cfg(use_graph=True)
+    eng = ZipageEngine(cfg)
+    torch.manual_seed(0)
+    params = [SamplingParams(max_tokens=40, ignore_eos=True, temperature=t) for t in (0.0, 0.8, 1.5)]
+    out = eng.generate(_prompts(3, [33, 64, 100], seed=9), params)
+    for o in out:
+        assert len(o["token_ids"]) == 40 and all(0 <= t < 503 for t in o["token_ids"])
+    # greedy request of the mixed batch equals a greedy-only run of the same prompt
+    solo, ref = _generate(_cfg(use_graph=False), _prompts(3, [33, 64, 100], seed=9)[:1], 40)
+    assert out[0]["token_ids"][:1] == ref[0]["token_ids"][:1]
+
+
+def test_prefix_cache_shares_pages_between_equal_prompts(dev):
+    """Two requests with the same first page: the second prefill reuses the page (refcount 2),
+    attends to it through the block table, and everything is released at the end."""
+    from zipage_amd.engine import SamplingParams, ZipageEngine
+    base = _prompts(1, [300], seed=11)[0]
+    other = base[:256] + _prompts(1, [50], seed=12)[0]
+    cfg = _cfg(use_graph=False, enable_prefix_cache=True, max_num_batched_tokens=320)
+    eng = ZipageEngine(cfg)
+    seen = {}
+    orig = eng.runner.run_prefill
+
+    def hooked(seqs):
+        for s in seqs:
+            seen[s.request_id] = (list(s.block_table), s.num_cached_tokens)
+        return orig(seqs)
+
+    eng.runner.run_prefill = hooked
+    out = eng.generate([base, other], SamplingParams(max_tokens=20, ignore_eos=True))
+    (t0, c0), (t1, c1) = [seen[k] for k in sorted(seen)]
+    assert c0 == 0 and c1 == 256 and t0[0] == t1[0] and t0[1] != t1[1]
+    assert all(len(o["token_ids"]) == 20 for o in out)
+    # the shared first page gives the second request the same first token as a run without sharing
+    solo, ref = _generate(_cfg(use_graph=False), [other], 20)
+    assert out[1]["token_ids"][0] == ref[0]["token_ids"][0]
+    pool = eng.scheduler.pool
+    assert pool.num_free == cfg.num_kvcache_blocks and not pool.refcount.any()

@@ -182,7 +182,7 @@ class ModelRunner:
         pinned, slot = self.ring.next()
         pinned[:words].numpy()[:] = packed
         with torch.cuda.stream(self.run_stream):
-            t = torch.tensor(temps, device=self.device) if any(temps) else None
+            t = torch.tensor(temps + [0.0] * (Bp - B), device=self.device) if any(temps) else None
             if graph:
                 g, sbuf, hidden = self._graph(Bp, TW)
                 sbuf.copy_(pinned[:words], non_blocking=True)
