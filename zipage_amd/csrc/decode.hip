@@ -1,7 +1,8 @@
 // The two cache-side kernels of the decode step that surround the compression path:
 // scattering the new token's K/V into the paged cache, and single-query attention over a
-// sequence's pages.  Both are HBM-streaming kernels (the decode step reads every cached K and V
-// once): 16 lanes own one 256-byte head vector, four token rows per wave instruction.
+// sequence's pages.  Both are HBM-streaming kernels: the decode step reads every cached K and V
+// exactly once, so the attention kernel is organised around 16-byte loads that cover whole
+// 128-byte lines of a (token, kv head) vector and around packed 16-bit dot products.
 #include "common.h"
 #include <math.h>
 

@@ -33,6 +33,11 @@ class ZipageEngine:
     # ------------------------------------------------------------------ requests
     def add_request(self, token_ids: list[int], params: SamplingParams | None = None) -> Sequence:
         seq = Sequence(token_ids, params or SamplingParams(), self.cfg.kvcache_block_size)
+        cfg = self.cfg
+        if not 0 < len(seq) <= min(cfg.max_num_batched_tokens, cfg.max_model_len):
+            raise ValueError(f"prompt of {len(seq)} tokens: need 1..{min(cfg.max_num_batched_tokens, cfg.max_model_len)}")
+        if seq.num_blocks > cfg.num_kvcache_blocks:
+            raise ValueError(f"prompt needs {seq.num_blocks} pages, the pool has {cfg.num_kvcache_blocks}")
         self.runner.reserve_token_log(seq.params.max_tokens + 1)
         self.scheduler.add(seq)
         return seq
@@ -120,9 +125,14 @@ class ZipageEngine:
         seqs = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
         step = self.async_step if self.cfg.enable_async_compress else self.step
         dev = self.runner.device
+        idle = 0
         while not self.is_finished():
             t0 = perf_counter()
             n = step()
+            idle = idle + 1 if n == 0 else 0
+            if idle > 10000:
+                raise RuntimeError("scheduler stalled: no sequence can get a page or a query row "
+                                   f"({self.scheduler.pool.num_free} pages free)")
             if n > 0:
                 torch.cuda.synchronize(dev)       # prefill is timed on its own
                 self.stats["prefill_s"] += perf_counter() - t0

@@ -83,8 +83,11 @@ class ModelRunner:
 
     def reserve_token_log(self, max_tokens: int):
         if self.token_log.shape[1] < max_tokens:
-            self.token_log = torch.zeros(self.cfg.max_concurrency + 1, max_tokens,
-                                         dtype=torch.int32, device=self.device)
+            old = self.token_log
+            with torch.cuda.stream(self.run_stream):   # ordered after the steps that wrote `old`
+                self.token_log = torch.zeros(self.cfg.max_concurrency + 1, max_tokens,
+                                             dtype=torch.int32, device=self.device)
+                self.token_log[:, :old.shape[1]] = old
             self._graphs.clear()
 
     # ------------------------------------------------------------------ step inputs
