@@ -301,8 +301,12 @@ __device__ __forceinline__ void split8(const float* x, bf16x8_t& hi, bf16x8_t& l
   }
 }
 
-template <typename T, bool RAW>
-__global__ __launch_bounds__(kThreads, 2) void gram_split_kernel(GramArgs p) {
+// NW waves per workgroup: every wave owns one 32-row block of the row page per round, so with 8
+// waves a 256-token page needs a single pass over the column tiles (they are normalised and split
+// once instead of twice).
+template <typename T, bool RAW, int NW>
+__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gram_split_kernel(GramArgs p) {
+  constexpr int kThreads = NW * 64, kWaves = NW;   // shadow the file-wide 4-wave constants
   static_assert(T::bytes == 2, "split path is for 16-bit caches");
   constexpr int PIECES = kDmax / 8;                 // 16-byte pieces per full key row
   constexpr int ROWS_PER_IT = kThreads / PIECES;    // 16
@@ -734,6 +738,15 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
       cval[t] = ok ? ws_val[base + t] : 0.f;
     }
     __syncthreads();
+    // Claims usually land on few rows: mark them, and only marked rows scan the claim list.
+    // The mark lives in x[], which the row's own value overwrites below.
+    for (int t = threadIdx.x; t < Tn; t += kThreads) x[t] = 0.f;
+    __syncthreads();
+    for (int t = threadIdx.x; t < Tn; t += kThreads) {
+      const int c = ccol[t];
+      if (c >= 0 && c < Tn) x[c] = 1.f;   // benign race: every writer stores the same value
+    }
+    __syncthreads();
   }
   float mloc = -INFINITY;
   for (int t = threadIdx.x; t < Tn; t += kThreads) {
@@ -743,8 +756,10 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
       const int pid = page_is_pad(c) ? -1 : page_id(c);
       if (pid >= 0 && pid < num_pages) {
         float corr = 0.f;
-        for (int j = 0; j < Tn; ++j)
-          if (ccol[j] == t) corr += cval[j];
+        if (x[t] != 0.f) {
+          for (int j = 0; j < Tn; ++j)
+            if (ccol[j] == t) corr += cval[j];
+        }
         r = Elem<T>::rnd(ws_sum[base + t] - corr);
       } else {
         r = -INFINITY;
@@ -808,13 +823,15 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
   }
   if constexpr (T::bytes == 2) {
     const size_t smem = 4 * (size_t)TN * ROWH + tail;
+    const bool wide = a.BS / 32 > kWaves;   // more row blocks than 4 waves: use 8 and halve the passes
+    const void* fn = wide ? (const void*)gram_split_kernel<T, RAW, 8> : (const void*)gram_split_kernel<T, RAW, 4>;
     if (smem > 64 * 1024 &&
-        hipFuncSetAttribute((const void*)gram_split_kernel<T, RAW>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+        hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
       zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
       return ZP_EHIP;
     }
-    hipLaunchKernelGGL((gram_split_kernel<T, RAW>), grid, dim3(kThreads), smem, st, a);
+    if (wide) hipLaunchKernelGGL((gram_split_kernel<T, RAW, 8>), grid, dim3(512), smem, st, a);
+    else hipLaunchKernelGGL((gram_split_kernel<T, RAW, 4>), grid, dim3(kThreads), smem, st, a);
   } else {
     const size_t smem = sizeof(float) * 2 * TN * ROWF + tail;
     if (smem > 64 * 1024 &&
