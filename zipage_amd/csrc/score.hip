@@ -28,7 +28,7 @@
 namespace {
 
 #ifndef ZP_SCORE_WAVES
-#define ZP_SCORE_WAVES 8
+#define ZP_SCORE_WAVES 4
 #endif
 constexpr int kWaves = ZP_SCORE_WAVES;  // waves per workgroup (4 or 8)
 constexpr int kThreads = kWaves * 64;
