@@ -31,6 +31,12 @@ namespace {
 #define ZP_SCORE_WAVES 4
 #endif
 constexpr int kWaves = ZP_SCORE_WAVES;  // waves per workgroup (4 or 8)
+#ifndef ZP_SCORE_TN16
+#define ZP_SCORE_TN16 (32 * kWaves)     // tokens per K tile for 16-bit caches
+#endif
+#ifndef ZP_SCORE_OCC
+#define ZP_SCORE_OCC 2                  // workgroups per CU the 16-bit kernel is compiled for
+#endif
 constexpr int kThreads = kWaves * 64;
 constexpr int kRowWaves = 4;   // most waves along the query-row axis; the other factor splits tokens.
                                // Fewer row blocks (small window x group) use 2 or 1 row waves so
@@ -47,14 +53,14 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 template <typename T> struct Mma;
 template <> struct Mma<BF16> {
   typedef bf16x8_t Frag;
-  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = 32 * kWaves, ROWB = kDmax * 2 + 16;
+  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = ZP_SCORE_TN16, ROWB = kDmax * 2 + 16;
   __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
 };
 template <> struct Mma<F16> {
   typedef f16x8_t Frag;
-  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = 32 * kWaves, ROWB = kDmax * 2 + 16;
+  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = ZP_SCORE_TN16, ROWB = kDmax * 2 + 16;
   __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
@@ -125,7 +131,7 @@ __device__ __forceinline__ float exp_neg(float x) {
 }
 
 template <typename T, bool LOGITS>
-__global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? 2 : 1)) void score_kernel(ScoreArgs p) {
+__global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_OCC : 1)) void score_kernel(ScoreArgs p) {
   typedef Mma<T> M;
   typedef typename M::Frag Frag;
   constexpr int TN = M::TN, ROWB = M::ROWB, KS = M::KS;
