@@ -37,6 +37,8 @@ def _ref_decode(q, k_cache, v_cache, ctx, tables, scale):
     (16, 8, 128, 256, 9, 3),      # Qwen3-0.6B
     (8, 8, 64, 16, 7, 4),         # no GQA, small pages
     (16, 2, 128, 32, 5, 2),       # group of 8
+    (32, 8, 128, 256, 40, 3),     # 10 240-token table: walked in slices with rescaled accumulators
+    (16, 2, 64, 256, 24, 2),      # sliced, group of 8
 ])
 def test_paged_decode_attention(dev, dtype, Hq, Hkv, D, BS, NB, B):
     from zipage_amd.layers import paged_decode_attention

@@ -71,6 +71,7 @@ struct DecodeArgs {
   void* out;           // (B, Hq, D)
   int B, Hq, Hkv, G, D, BS, NB, num_pages;
   int bs_shift;        // log2(BS) when BS is a power of two, else -1
+  int chunk;           // tokens per slice when the context is walked in slices (multiple of 128)
   int64_t k_sp, v_sp;  // page strides in elements
   float scale;
 };
@@ -90,8 +91,8 @@ constexpr int kUnroll = 4;             // rows per lane group and loop trip (mus
 //           packed in pairs (token t, token t + 32) over the logit word of t
 //   pass 3: out += p.v with two tokens per dot2 (the pair above), fp32 accumulate; the row
 //           groups are summed at the end and scaled by 1 / sum(p).
-template <typename T, int G>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(G <= 4 ? 4 : 2, 4))) void paged_decode_kernel(DecodeArgs p) {
+template <typename T, int G, bool CHUNKED>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(G <= 4 && !CHUNKED ? 4 : 2, 4))) void paged_decode_kernel(DecodeArgs p) {
   extern __shared__ __align__(16) float lds[];
   __shared__ float red[kWaves * G];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -99,7 +100,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(G <= 4
   const int h = blockIdx.x % p.Hkv, b = blockIdx.x / p.Hkv;
   int Tn = p.ctx[b];
   Tn = max(0, min(Tn, p.NB * p.BS));
-  const int Tpad = (p.NB * p.BS + 63) & ~63;
+  const int Tpad = CHUNKED ? p.chunk : ((p.NB * p.BS + 63) & ~63);   // LDS row of one head's logits
   float* logit = lds;                            // [G][Tpad]
   uint32_t* pw = (uint32_t*)lds;                 // packed p pairs over the same words
   const int pieces = p.D / 8;                    // 16-byte pieces per head vector (<= 16)
@@ -124,143 +125,171 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(G <= 4
     return cache + (int64_t)pages_lds[pg] * page_stride * 2 + (int64_t)slot * row;
   };
 
-  // ---- pass 1: logits
-  {
-    u32x4 qa[G], qb[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      const char* qp = p.q + (((int64_t)b * p.Hq + h * G + g) * p.D) * 2;
-      qa[g] = onA ? *(const u32x4*)(qp + sub * 16) : zero4;
-      qb[g] = onB ? *(const u32x4*)(qp + (sub + 8) * 16) : zero4;
-    }
-    // rows of the next trip are requested before the current ones are consumed
-    u32x4 ka[kUnroll], kb[kUnroll], na[kUnroll], nb[kUnroll];
-    auto fetch_k = [&](int t0, u32x4* a, u32x4* bq) {
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        const char* base = row_base(p.k, p.k_sp, t0 + u * kGroups + grp);
-        a[u] = ZP_DEC_LOAD((const u32x4*)(base + offA));
-        bq[u] = ZP_DEC_LOAD((const u32x4*)(base + offB));
-      }
-    };
-    if (Tn > 0) fetch_k(0, ka, kb);
-    for (int t0 = 0; t0 < Tn; t0 += kGroups * kUnroll) {
-      const bool more = t0 + kGroups * kUnroll < Tn;
-      if (more) fetch_k(t0 + kGroups * kUnroll, na, nb);
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        const int t = t0 + u * kGroups + grp;
-        float mine = 0.f;
-#pragma unroll
-        for (int g = 0; g < G; ++g) {
-          float a = 0.f;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) a = dot2<T>(ka[u][i], qa[g][i], a);
-#pragma unroll
-          for (int i = 0; i < 4; ++i) a = dot2<T>(kb[u][i], qb[g][i], a);
-          a = group8_sum(a);
-          mine = (sub == g) ? a : mine;
-        }
-        if (sub < G && t < Tn) logit[sub * Tpad + t] = mine * p.scale;
-      }
-      if (more) {
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) { ka[u] = na[u]; kb[u] = nb[u]; }
-      }
-    }
-  }
-  __syncthreads();
-  // ---- pass 2: softmax statistics per head, p packed in pairs (t, t + 32)
-  float inv[G];
-  {
-    float mx[G];
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float m = -INFINITY;
-      for (int t = tid; t < Tn; t += kThreads) m = fmaxf(m, logit[g * Tpad + t]);
-      m = wave_max(m);
-      if (lane == 0) red[wave * G + g] = m;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float m = red[g];
-      for (int w = 1; w < kWaves; ++w) m = fmaxf(m, red[w * G + g]);
-      mx[g] = m;
-    }
-    __syncthreads();
-    const int npairs = ((Tn + 63) >> 6) * 32;
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float s = 0.f;
-      for (int pi = tid; pi < npairs; pi += kThreads) {
-        const int t = (pi >> 5) * 64 + (pi & 31);
-        // each token belongs to exactly one pair, so the packed word can overwrite logit[t]
-        const float e0 = t < Tn ? __expf(logit[g * Tpad + t] - mx[g]) : 0.f;
-        const float e1 = t + 32 < Tn ? __expf(logit[g * Tpad + t + 32] - mx[g]) : 0.f;
-        s += e0 + e1;
-        pw[g * Tpad + t] = pack2<T>(e0, e1);
-      }
-      s = wave_sum(s);
-      if (lane == 0) red[wave * G + g] = s;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int g = 0; g < G; ++g) {
-      float s = 0.f;
-      for (int w = 0; w < kWaves; ++w) s += red[w * G + g];
-      inv[g] = s > 0.f ? 1.f / s : 0.f;
-    }
-  }
-  // ---- pass 3: P.V, two tokens per dot2.  Sixteen lanes per row here (one 16-byte piece each),
-  // which halves the accumulators a lane carries; a trip covers two 64-token blocks, and row
-  // group `g16` takes the pairs j = g16 and j = g16 + 16 of each.
+  // accumulators of pass 3 (sixteen lanes per V row, one 16-byte piece each) and the running
+  // softmax statistics; with CHUNKED the context is walked in slices of p.chunk tokens and both
+  // are carried from slice to slice (rescaled when the maximum grows)
   const int g16 = tid >> 4, s16 = tid & 15;
   const bool onV = s16 < pieces;
   const int64_t offV = (int64_t)h * p.D * 2 + (onV ? s16 * 16 : 0);
-  float acc[G][8];
+  float acc[G][8], m_run[G], l_run[G];
 #pragma unroll
-  for (int g = 0; g < G; ++g)
+  for (int g = 0; g < G; ++g) {
+    m_run[g] = -INFINITY;
+    l_run[g] = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[g][i] = 0.f;
-  constexpr int kPairs = 4;
-  u32x4 vx[kPairs], vy[kPairs], nx[kPairs], ny[kPairs];
-  auto fetch_v = [&](int t0, u32x4* x, u32x4* y) {
+  }
+  auto slice = [&](const int c0, const int Tc) {   // Tc tokens from c0; LDS indices are slice-local
+    // ---- pass 1: logits
+    {
+      u32x4 qa[G], qb[G];
 #pragma unroll
-    for (int u = 0; u < kPairs; ++u) {
-      const int t = t0 + (u >> 1) * 64 + (u & 1) * 16 + g16;
-      x[u] = ZP_DEC_LOAD((const u32x4*)(row_base(p.v, p.v_sp, t) + offV));
-      y[u] = ZP_DEC_LOAD((const u32x4*)(row_base(p.v, p.v_sp, t + 32) + offV));
-    }
-  };
-  if (Tn > 0) fetch_v(0, vx, vy);
-  for (int t0 = 0; t0 < Tn; t0 += 16 * kPairs * 2) {
-    const bool more = t0 + 16 * kPairs * 2 < Tn;
-    if (more) fetch_v(t0 + 16 * kPairs * 2, nx, ny);
+      for (int g = 0; g < G; ++g) {
+        const char* qp = p.q + (((int64_t)b * p.Hq + h * G + g) * p.D) * 2;
+        qa[g] = onA ? *(const u32x4*)(qp + sub * 16) : zero4;
+        qb[g] = onB ? *(const u32x4*)(qp + (sub + 8) * 16) : zero4;
+      }
+      // rows of the next trip are requested before the current ones are consumed
+      u32x4 ka[kUnroll], kb[kUnroll], na[kUnroll], nb[kUnroll];
+      auto fetch_k = [&](int t0, u32x4* a, u32x4* bq) {
 #pragma unroll
-    for (int u = 0; u < kPairs; ++u) {
-      const int t = t0 + (u >> 1) * 64 + (u & 1) * 16 + g16;  // partner is t + 32
-      if (t < Tn) {
-        uint32_t pp[G];
+        for (int u = 0; u < kUnroll; ++u) {
+          const char* base = row_base(p.k, p.k_sp, c0 + t0 + u * kGroups + grp);
+          a[u] = ZP_DEC_LOAD((const u32x4*)(base + offA));
+          bq[u] = ZP_DEC_LOAD((const u32x4*)(base + offB));
+        }
+      };
+      fetch_k(0, ka, kb);
+      for (int t0 = 0; t0 < Tc; t0 += kGroups * kUnroll) {
+        const bool more = t0 + kGroups * kUnroll < Tc;
+        if (more) fetch_k(t0 + kGroups * kUnroll, na, nb);
 #pragma unroll
-        for (int g = 0; g < G; ++g) pp[g] = pw[g * Tpad + t];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint32_t lo = __builtin_amdgcn_perm(vy[u][i], vx[u][i], 0x05040100u);  // (x.lo16, y.lo16)
-          const uint32_t hi = __builtin_amdgcn_perm(vy[u][i], vx[u][i], 0x07060302u);  // (x.hi16, y.hi16)
+        for (int u = 0; u < kUnroll; ++u) {
+          const int t = t0 + u * kGroups + grp;
+          float mine = 0.f;
 #pragma unroll
           for (int g = 0; g < G; ++g) {
-            acc[g][2 * i] = dot2<T>(lo, pp[g], acc[g][2 * i]);
-            acc[g][2 * i + 1] = dot2<T>(hi, pp[g], acc[g][2 * i + 1]);
+            float a = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a = dot2<T>(ka[u][i], qa[g][i], a);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a = dot2<T>(kb[u][i], qb[g][i], a);
+            a = group8_sum(a);
+            mine = (sub == g) ? a : mine;
           }
+          if (sub < G && t < Tc) logit[sub * Tpad + t] = mine * p.scale;
+        }
+        if (more) {
+#pragma unroll
+          for (int u = 0; u < kUnroll; ++u) { ka[u] = na[u]; kb[u] = nb[u]; }
         }
       }
     }
-    if (more) {
+    __syncthreads();
+    // ---- pass 2: softmax statistics per head, p packed in pairs (t, t + 32)
+    {
+      float mx[G];
 #pragma unroll
-      for (int u = 0; u < kPairs; ++u) { vx[u] = nx[u]; vy[u] = ny[u]; }
+      for (int g = 0; g < G; ++g) {
+        float m = -INFINITY;
+        for (int t = tid; t < Tc; t += kThreads) m = fmaxf(m, logit[g * Tpad + t]);
+        m = wave_max(m);
+        if (lane == 0) red[wave * G + g] = m;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float m = red[g];
+        for (int w = 1; w < kWaves; ++w) m = fmaxf(m, red[w * G + g]);
+        mx[g] = CHUNKED ? fmaxf(m, m_run[g]) : m;
+      }
+      __syncthreads();
+      const int npairs = ((Tc + 63) >> 6) * 32;
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float s = 0.f;
+        for (int pi = tid; pi < npairs; pi += kThreads) {
+          const int t = (pi >> 5) * 64 + (pi & 31);
+          // each token belongs to exactly one pair, so the packed word can overwrite logit[t]
+          const float e0 = t < Tc ? __expf(logit[g * Tpad + t] - mx[g]) : 0.f;
+          const float e1 = t + 32 < Tc ? __expf(logit[g * Tpad + t + 32] - mx[g]) : 0.f;
+          s += e0 + e1;
+          pw[g * Tpad + t] = pack2<T>(e0, e1);
+        }
+        s = wave_sum(s);
+        if (lane == 0) red[wave * G + g] = s;
+      }
+      __syncthreads();
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        float s = 0.f;
+        for (int w = 0; w < kWaves; ++w) s += red[w * G + g];
+        if (CHUNKED) {
+          // earlier slices were accumulated against a smaller maximum: bring them to this one
+          const float f = __expf(m_run[g] - mx[g]);   // exp(-inf) = 0 on the first slice
+          l_run[g] = l_run[g] * f + s;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc[g][i] *= f;
+        } else {
+          l_run[g] = s;
+        }
+        m_run[g] = mx[g];
+      }
     }
+    // ---- pass 3: P.V, two tokens per dot2; a trip covers two 64-token blocks, and row group
+    // `g16` takes the pairs j = g16 and j = g16 + 16 of each.
+    {
+      constexpr int kPairs = 4;
+      u32x4 vx[kPairs], vy[kPairs], nx[kPairs], ny[kPairs];
+      auto fetch_v = [&](int t0, u32x4* x, u32x4* y) {
+#pragma unroll
+        for (int u = 0; u < kPairs; ++u) {
+          const int t = c0 + t0 + (u >> 1) * 64 + (u & 1) * 16 + g16;
+          x[u] = ZP_DEC_LOAD((const u32x4*)(row_base(p.v, p.v_sp, t) + offV));
+          y[u] = ZP_DEC_LOAD((const u32x4*)(row_base(p.v, p.v_sp, t + 32) + offV));
+        }
+      };
+      fetch_v(0, vx, vy);
+      for (int t0 = 0; t0 < Tc; t0 += 16 * kPairs * 2) {
+        const bool more = t0 + 16 * kPairs * 2 < Tc;
+        if (more) fetch_v(t0 + 16 * kPairs * 2, nx, ny);
+#pragma unroll
+        for (int u = 0; u < kPairs; ++u) {
+          const int t = t0 + (u >> 1) * 64 + (u & 1) * 16 + g16;  // partner is t + 32
+          if (t < Tc) {
+            uint32_t pp[G];
+#pragma unroll
+            for (int g = 0; g < G; ++g) pp[g] = pw[g * Tpad + t];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const uint32_t lo = __builtin_amdgcn_perm(vy[u][i], vx[u][i], 0x05040100u);  // (x.lo16, y.lo16)
+              const uint32_t hi = __builtin_amdgcn_perm(vy[u][i], vx[u][i], 0x07060302u);  // (x.hi16, y.hi16)
+#pragma unroll
+              for (int g = 0; g < G; ++g) {
+                acc[g][2 * i] = dot2<T>(lo, pp[g], acc[g][2 * i]);
+                acc[g][2 * i + 1] = dot2<T>(hi, pp[g], acc[g][2 * i + 1]);
+              }
+            }
+          }
+        }
+        if (more) {
+#pragma unroll
+          for (int u = 0; u < kPairs; ++u) { vx[u] = nx[u]; vy[u] = ny[u]; }
+        }
+      }
+    }
+  };
+  if constexpr (CHUNKED) {
+    for (int c0 = 0; c0 < Tn; c0 += p.chunk) {
+      slice(c0, min(p.chunk, Tn - c0));
+      __syncthreads();   // the next slice's logits overwrite this slice's p
+    }
+  } else {
+    if (Tn > 0) slice(0, Tn);   // one pass: nothing is carried, the accumulators start at pass 3
   }
+  float inv[G];
+#pragma unroll
+  for (int g = 0; g < G; ++g) inv[g] = l_run[g] > 0.f ? 1.f / l_run[g] : 0.f;
   // sum the 4 row groups of each wave (lanes with equal piece), then the waves through LDS
 #pragma unroll
   for (int g = 0; g < G; ++g)
@@ -289,24 +318,29 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(G <= 4
   }
 }
 
+// Contexts whose logits fit 72 KB of LDS (4608 tokens at a group of 4) run in one slice; longer
+// ones (a long prompt before its first compression) are walked in slices of 2048 tokens.
+constexpr int kSingleSliceBytes = 72 * 1024;
+constexpr int kSliceTokens = 2048;
+
 template <typename T, int G>
-int launch_decode(const DecodeArgs& a, hipStream_t st) {
+int launch_decode(DecodeArgs a, hipStream_t st) {
   const int Tpad = (a.NB * a.BS + 63) & ~63;
-  size_t smem = sizeof(float) * (size_t)G * Tpad;
   const size_t part = sizeof(float) * kWaves * G * 128;
+  const bool chunked = sizeof(float) * (size_t)G * Tpad > kSingleSliceBytes;
+  a.chunk = chunked ? kSliceTokens : 0;
+  size_t smem = sizeof(float) * (size_t)G * (chunked ? kSliceTokens : Tpad);
   if (part > smem) smem = part;
-  if (smem > 150 * 1024) {
-    zp_set_error("paged_decode_attention: %d cached tokens x %d heads exceed LDS", a.NB * a.BS, G);
-    return ZP_EUNSUPPORTED;
-  }
+  const void* fn = chunked ? (const void*)paged_decode_kernel<T, G, true>
+                           : (const void*)paged_decode_kernel<T, G, false>;
   if (smem > 64 * 1024 &&
-      hipFuncSetAttribute((const void*)paged_decode_kernel<T, G>,
-                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+      hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
     zp_set_error("paged_decode_attention: cannot reserve %zu bytes of LDS", smem);
     return ZP_EHIP;
   }
-  hipLaunchKernelGGL((paged_decode_kernel<T, G>), dim3((unsigned)(a.B * a.Hkv)), dim3(kThreads), smem,
-                     st, a);
+  const dim3 grid((unsigned)(a.B * a.Hkv));
+  if (chunked) hipLaunchKernelGGL((paged_decode_kernel<T, G, true>), grid, dim3(kThreads), smem, st, a);
+  else hipLaunchKernelGGL((paged_decode_kernel<T, G, false>), grid, dim3(kThreads), smem, st, a);
   ZP_LAUNCH_CHECK();
   return ZP_OK;
 }
