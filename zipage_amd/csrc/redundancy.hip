@@ -635,22 +635,30 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
         }
       }
       const int cslot = cb * 32 + col;
+      if (cb == rb) {   // the diagonal (a key against itself) only lives in this block
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if ((r >> 2) * 8 + half * 4 + (r & 3) == col) acc[r] = 0.f;
+      }
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-        float s = acc[r];
-        if (rslot == cslot) s = 0.f;
+        const float s = acc[r];
         rsum[r] += s;
         if (s > p.threshold) { ccol[r] = cslot; cval[r] = s; }
       }
     }
+    // most waves see no entry over the threshold: then the (column, value) reduction is skipped
+    bool mine = false;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mine |= ccol[r] >= 0;
+    const bool any_claim = __any(mine);
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       float s = rsum[r];
       int c = ccol[r];
       float v = cval[r];
       s = half_sum(s);
-      last_claim_reduce(c, v);
+      if (any_claim) last_claim_reduce(c, v);
       if (col == 0) {
         const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
         l_sum[rslot] = s;
