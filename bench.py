@@ -133,7 +133,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--config", type=int, default=2, choices=[2, 4, 5],
-                    help="BASELINE config (1-based as in SURVEY): 2 = 64 ragged sequences, one "
+                    help="workload, numbered from 1 as in BASELINE.json: 2 = 64 ragged sequences, one "
                          "layer (default, the headline line); 4 = 256 sequences with shared "
                          "prefixes and copy-on-write targets, 36 layers run one layer at a time "
                          "over one page pool; 5 = the end-to-end decode case alone")
