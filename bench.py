@@ -148,6 +148,9 @@ def main():
     ap.add_argument("--ragged-prompts", action="store_true",
                     help="end-to-end leg: prompt lengths uniform in [P/2, 3P/2] so sequences reach "
                          "their budget on different steps")
+    ap.add_argument("--separate-select-stages", action="store_true",
+                    help="run pooling, the mask epilogue and top-k as three launches (timed under "
+                         "the reference's stage names) instead of the one-launch selection")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", type=int, default=64)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -202,7 +205,8 @@ def main():
     def step(timer=None):
         for _ in range(layers):
             compress_layers(wl.k, wl.v, wl.q, wl.score_cache, wl.query_ids, wl.block_tables,
-                            wl.compressed, wl.targets, cfg, timer=timer)
+                            wl.compressed, wl.targets, cfg, timer=timer,
+                            fused_select=not args.separate_select_stages)
 
     if args.calibrate_copy:
         src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")

@@ -142,6 +142,26 @@ int zp_score_epilogue(void* scores, const void* redundancy, const int32_t* block
 int zp_topk_mask(const void* scores, uint8_t* flag_out, int32_t rows, int32_t T, int32_t k,
                  int32_t dtype, void* stream);
 
+/* The selection stages of one layer chunk in one pass per score row (no counterpart as a
+ * single function in the reference, which runs them inline in the runner):
+ *   zipage/engine/model_runner.py:499-530  pooling (pool_kernel_size > 1; see zp_pool_scores)
+ *   zipage/engine/model_runner.py:551-559  red /= max_T (max_norm_red);
+ *                                          scores*lambda - red*(1-lambda)  (redundancy != NULL)
+ *   zipage/engine/model_runner.py:565-578  first sink_len tokens -> +inf
+ *   zipage/kernel/window_mask.py:47-72     last `window` slots of the last page -> +inf
+ *   zipage/engine/model_runner.py:592-593  pad pages -> -inf               (mask_pad)
+ *   zipage/engine/model_runner.py:594-600, zipage/kernel/utils.py:21-36    top-k keep flag
+ * Results are bit-identical to zp_pool_scores + zp_score_epilogue + zp_topk_mask run one
+ * after the other.  scores (L, B, Hkv, NB*BS) is read only unless scores_out == scores;
+ * scores_out (same shape, may be NULL) receives the post-processed scores;
+ * flag_out (L, B, Hkv, NB*BS) bytes, exactly k ones per row, ties to the lowest index. */
+int zp_select_topk(const void* scores, void* scores_out, const void* redundancy,
+                   uint8_t* flag_out, const int32_t* block_table, const uint8_t* compressed,
+                   int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
+                   int32_t pool_kernel_size, int32_t continues_pooling, int32_t pool_mode,
+                   int32_t max_norm_red, double redudancy_lambda, int32_t sink_len,
+                   int32_t window, int32_t mask_pad, int32_t k, int32_t dtype, void* stream);
+
 /* compress_kv(key, value, flag, block_table, target_block_table)
  * zipage/kernel/compress_kv.py:103-141 (kernel :8-100).
  * key/value (L, num_pages, BS, Hkv, D) with the given element strides (head_dim stride

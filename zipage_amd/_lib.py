@@ -37,6 +37,8 @@ SIGNATURES = {
     "zp_score_epilogue": [ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32, f64, i32, i32, i32,
                           i32, ptr],
     "zp_topk_mask": [ptr, ptr, i32, i32, i32, i32, ptr],
+    "zp_select_topk": [ptr, ptr, ptr, ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32, i32, i32,
+                       f64, i32, i32, i32, i32, i32, ptr],
     "zp_compress_kv": [ptr, ptr, ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32, i32,
                        i64, i64, i64, i64, i64, i64, i64, i64, i32, ptr],
     "zp_compress_score": [ptr, ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32, i64, i64, i64,

@@ -19,12 +19,16 @@ from zipage_amd.kernel.global_score import global_score
 from zipage_amd.kernel.lightning_redudancy_score import lightning_redudancy_score
 from zipage_amd.kernel.pooling import pool_scores
 from zipage_amd.kernel.raw_redudancy_score import raw_redudancy_score
+from zipage_amd.kernel.select import MAX_ROW_TOKENS, select_topk
 from zipage_amd.kernel.utils import topk_mask
 from zipage_amd.kernel.window_mask import score_epilogue
 
 # stage names as the reference records them (model_runner.py:424-429,624-630)
 STAGES = ("attention_score", "global_score", "pooling", "redudancy_score", "attention_sink",
           "window_mask", "topk_mask", "compress_kv", "compress_global_score")
+# pooling, combine, sink / window / pad masks and top-k run as one launch unless a caller asks
+# for the separate stages; the timer then books them under this one name
+FUSED_SELECT_STAGE = "pooling+window_mask+topk_mask"
 
 
 @dataclass
@@ -81,7 +85,7 @@ class StageTimer:
 
 def compress_layers(k_cache, v_cache, query_cache, score_cache, query_ids, block_tables,
                     compressed, target_block_tables, cfg: CompressConfig, timer=None,
-                    return_intermediates=False):
+                    return_intermediates=False, fused_select=True):
     """Score, select and compact one chunk of layers in place.
 
     k_cache/v_cache: (L, num_pages, BS, Hkv, D); query_cache: (L, max_seqs, W, Hq, D);
@@ -105,12 +109,6 @@ def compress_layers(k_cache, v_cache, query_cache, score_cache, query_ids, block
                               cfg.activate_method)
         t.stop(ev)
 
-    if cfg.enable_pooling:
-        ev = t.start("pooling")
-        scores = pool_scores(scores, compressed, cfg.pooling_size, cfg.continues_pooling,
-                             cfg.pooling_mode)
-        t.stop(ev)
-
     red = None
     if cfg.use_redudancy:
         ev = t.start("redudancy_score")
@@ -119,20 +117,40 @@ def compress_layers(k_cache, v_cache, query_cache, score_cache, query_ids, block
                  temperature=cfg.redudancy_temperature)
         t.stop(ev)
 
-    # combine + sink + window mask + pad mask: one fused pass (window_mask stage)
-    ev = t.start("window_mask")
-    score_epilogue(scores, block_tables, red,
-                   max_norm_red=cfg.use_redudancy and cfg.use_global_score and cfg.max_norm,
-                   redudancy_lambda=cfg.redudancy_lambda,
-                   sink_len=cfg.sink_len if cfg.use_attention_sink else 0,
-                   window=cfg.query_cache_len, mask_pad=True)
-    t.stop(ev)
-
-    ev = t.start("topk_mask")
     L, B, Hkv, NB, _ = scores.shape
-    flag = topk_mask(scores.view(L, B, Hkv, NB * BS), BS * cfg.budget_blocks)
-    flag = flag.view(L, B, Hkv, NB, BS)
-    t.stop(ev)
+    if fused_select and NB * BS <= MAX_ROW_TOKENS:
+        ev = t.start(FUSED_SELECT_STAGE)
+        out = select_topk(scores, block_tables, compressed, BS * cfg.budget_blocks,
+                          pooling_size=cfg.pooling_size if cfg.enable_pooling else 0,
+                          continues_pooling=cfg.continues_pooling, pooling_mode=cfg.pooling_mode,
+                          redundancy=red,
+                          max_norm_red=cfg.use_redudancy and cfg.use_global_score and cfg.max_norm,
+                          redudancy_lambda=cfg.redudancy_lambda,
+                          sink_len=cfg.sink_len if cfg.use_attention_sink else 0,
+                          window=cfg.query_cache_len, mask_pad=True,
+                          return_scores=return_intermediates)
+        flag, scores = out if return_intermediates else (out, scores)
+        t.stop(ev)
+    else:
+        if cfg.enable_pooling:
+            ev = t.start("pooling")
+            scores = pool_scores(scores, compressed, cfg.pooling_size, cfg.continues_pooling,
+                                 cfg.pooling_mode)
+            t.stop(ev)
+
+        # combine + sink + window mask + pad mask: one fused pass (window_mask stage)
+        ev = t.start("window_mask")
+        score_epilogue(scores, block_tables, red,
+                       max_norm_red=cfg.use_redudancy and cfg.use_global_score and cfg.max_norm,
+                       redudancy_lambda=cfg.redudancy_lambda,
+                       sink_len=cfg.sink_len if cfg.use_attention_sink else 0,
+                       window=cfg.query_cache_len, mask_pad=True)
+        t.stop(ev)
+
+        ev = t.start("topk_mask")
+        flag = topk_mask(scores.view(L, B, Hkv, NB * BS), BS * cfg.budget_blocks)
+        flag = flag.view(L, B, Hkv, NB, BS)
+        t.stop(ev)
 
     ev = t.start("compress_kv")
     compress_kv(k_cache, v_cache, flag, block_tables, target_block_tables)

@@ -86,6 +86,288 @@ __global__ __launch_bounds__(kThreads) void topk_mask_kernel(const void* __restr
   }
 }
 
+
+// ------------------------------------------------------------------ fused selection
+// Pooling, redundancy combine, sink / window / pad masks and the top-k of one score row in a
+// single pass.  The per-element arithmetic and its rounding points are those of pool_kernel
+// and epilogue_kernel, so the result equals running the three stages one after the other.
+struct SelectArgs {
+  const void* scores;
+  void* scores_out;         // may be null
+  const void* red;          // may be null
+  uint8_t* flag;
+  const int32_t* table;
+  const uint8_t* compressed;
+  int B, NB, BS, Hkv, ksize, continues, mode, norm_r;
+  float lam, one_minus_lam;
+  int sink_len, window, mask_pad, k, low_bit;
+};
+
+// Row -> LDS as fp32, 16 bytes per thread per step when the row allows it.
+template <typename T>
+__device__ __forceinline__ void stage_row(const void* __restrict__ src, int64_t base, int Tn,
+                                          float* __restrict__ row) {
+  constexpr int EPV = 16 / T::bytes;  // elements per 16-byte piece
+  const char* p = (const char*)src + base * T::bytes;
+  if ((Tn % EPV) == 0 && ((uintptr_t)p & 15) == 0) {
+    for (int c = threadIdx.x; c < Tn / EPV; c += kThreads) {
+      const vec16 v = ((const vec16*)p)[c];
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+      float* dst = row + c * EPV;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if constexpr (T::bytes == 4) {
+          dst[i] = __uint_as_float(w[i]);
+        } else {
+          const uint16_t lo = (uint16_t)(w[i] & 0xffffu), hi = (uint16_t)(w[i] >> 16);
+          dst[2 * i] = Elem<T>::ld(&lo, 0);
+          dst[2 * i + 1] = Elem<T>::ld(&hi, 0);
+        }
+      }
+    }
+  } else {
+    for (int t = threadIdx.x; t < Tn; t += kThreads) row[t] = Elem<T>::ld(src, base + t);
+  }
+}
+
+__device__ __forceinline__ float block_max_of(float m, float* max_lds) {
+  m = wave_max(m);
+  if (lane_id() == 0) max_lds[wave_id()] = m;
+  __syncthreads();
+  float r = max_lds[0];
+#pragma unroll
+  for (int i = 1; i < kWaves; ++i) r = fmaxf(r, max_lds[i]);
+  return r;
+}
+
+// Combine with the redundancy and apply the masks to one pooled value (epilogue_kernel's
+// per-element body).
+template <typename T>
+__device__ __forceinline__ float select_finish(const SelectArgs& p, float v, int t, int64_t base,
+                                               int code, int slot, float rmax) {
+  if (p.red) {
+    float rv = Elem<T>::ld(p.red, base + t);
+    if (p.norm_r) rv = Elem<T>::rnd(rv / rmax);
+    const float a = Elem<T>::rnd(v * p.lam);
+    const float c = Elem<T>::rnd(rv * p.one_minus_lam);
+    v = Elem<T>::rnd(a - c);
+  }
+  if (t < p.sink_len) v = INFINITY;
+  if (p.window > 0 && page_is_last(code) && slot >= p.BS - p.window) v = INFINITY;
+  if (p.mask_pad && page_is_pad(code)) v = -INFINITY;
+  if (p.scores_out) Elem<T>::st(p.scores_out, base + t, v);
+  return v;
+}
+
+// Flags staged in LDS by index-ordered owners, then written out coalesced.
+__device__ __forceinline__ void write_flags(const uint8_t* fl, uint8_t* __restrict__ flag,
+                                            int64_t base, int Tn) {
+  if ((Tn & 3) == 0 && ((uintptr_t)flag & 3) == 0) {
+    const uint32_t* src = (const uint32_t*)fl;
+    uint32_t* dst = (uint32_t*)(flag + base);
+    for (int t = threadIdx.x; t < Tn / 4; t += kThreads) dst[t] = src[t];
+  } else {
+    for (int t = threadIdx.x; t < Tn; t += kThreads) flag[base + t] = fl[t];
+  }
+}
+
+// Rows of at most 256 * PER tokens with a pooling window of at most 7: every thread owns a
+// contiguous, index-ordered chunk of PER tokens, reads the PER + 6 raw scores its windows
+// cover from LDS once and keeps its keys in registers, so each step of the bit search is
+// PER compares, one wave sum and one barrier.
+constexpr int kSelHalf = 3;
+template <typename T, int PER>
+__global__ __launch_bounds__(kThreads) void select_reg_kernel(SelectArgs p) {
+  extern __shared__ float row[];
+  __shared__ int slots[2][kWaves];
+  __shared__ int scan_lds[kWaves];
+  __shared__ float max_lds[kWaves];
+  const int tid = threadIdx.x;
+  const int Tn = p.NB * p.BS;
+  const int64_t r = blockIdx.x;
+  const int b = (int)((r / p.Hkv) % p.B);
+  const int64_t base = r * Tn;
+  const int32_t* trow = p.table + (int64_t)b * p.NB;
+
+  stage_row<T>(p.scores, base, Tn, row);
+  float rmax = 1.f;
+  if (p.red && p.norm_r) {
+    float m = -INFINITY;
+    for (int t = tid; t < Tn; t += kThreads) m = fmaxf(m, Elem<T>::ld(p.red, base + t));
+    rmax = block_max_of(m, max_lds);  // its barrier also publishes row[]
+  } else {
+    __syncthreads();
+  }
+
+  const int chunk = (Tn + kThreads - 1) / kThreads;  // <= PER
+  const int s0 = min(tid * chunk, Tn), s1 = min(s0 + chunk, Tn);
+  const bool pooled = p.ksize > 1 && (p.continues || p.compressed[b] == 0);
+  const int half = pooled ? p.ksize / 2 : 0;
+  const bool is_max = p.mode == ZP_POOL_MAX;
+  float win[PER + 2 * kSelHalf];
+#pragma unroll
+  for (int j = 0; j < PER + 2 * kSelHalf; ++j) {
+    const int idx = s0 - kSelHalf + j;
+    win[j] = (idx >= 0 && idx < Tn) ? row[idx] : (is_max ? -INFINITY : 0.f);
+  }
+  int j = s0 / p.BS, slot = s0 - j * p.BS;
+  int code = s0 < Tn ? trow[j] : -1;
+  uint32_t kreg[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    kreg[i] = 0u;  // below every real key
+    if (s0 + i < s1) {
+      float v = win[i + kSelHalf];
+      if (pooled) {
+        if (is_max) {
+#pragma unroll
+          for (int d = 1; d <= kSelHalf; ++d) {
+            if (d <= half) v = fmaxf(fmaxf(v, win[i + kSelHalf - d]), win[i + kSelHalf + d]);
+          }
+        } else {
+          float acc = 0.f;  // ascending index order, as pool_kernel adds
+#pragma unroll
+          for (int d = -kSelHalf; d <= kSelHalf; ++d) {
+            if (d >= -half && d <= half) acc += win[i + kSelHalf + d];
+          }
+          v = Elem<T>::rnd(acc / (float)p.ksize);
+        }
+      }
+      v = select_finish<T>(p, v, s0 + i, base, code, slot, rmax);
+      kreg[i] = score_key(v, p.low_bit);
+      if (++slot == p.BS) {
+        slot = 0;
+        ++j;
+        if (s0 + i + 1 < s1) code = trow[j];
+      }
+    }
+  }
+
+  uint32_t prefix = 0;
+  int pp = 0;
+  for (int bit = 31; bit >= p.low_bit; --bit) {
+    const uint32_t cand = prefix | (1u << bit);
+    int c = 0;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) c += kreg[i] >= cand ? 1 : 0;
+    if (block_count(c, slots[pp]) >= p.k) prefix = cand;
+    pp ^= 1;
+  }
+  // prefix is the k-th largest key; keep everything above it and the first few equal to it
+  int cg = 0, ce = 0;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    cg += kreg[i] > prefix ? 1 : 0;
+    ce += (s0 + i < s1 && kreg[i] == prefix) ? 1 : 0;
+  }
+  const int need_eq = p.k - block_count(cg, slots[pp]);
+  int inc = ce;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    int t = __shfl_up(inc, o, 64);
+    if (lane_id() >= o) inc += t;
+  }
+  if (lane_id() == 63) scan_lds[wave_id()] = inc;
+  __syncthreads();  // every thread has long finished reading row[] as floats
+  int rank = inc - ce;
+  for (int i = 0; i < wave_id(); ++i) rank += scan_lds[i];
+  uint8_t* fl = (uint8_t*)row;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    if (s0 + i < s1) {
+      uint8_t f = kreg[i] > prefix ? 1 : 0;
+      if (kreg[i] == prefix) { f = rank < need_eq ? 1 : 0; ++rank; }
+      fl[s0 + i] = f;
+    }
+  }
+  __syncthreads();
+  write_flags(fl, p.flag, base, Tn);
+}
+
+// Any row that fits LDS twice (raw scores + keys), any odd pooling window.
+template <typename T>
+__global__ __launch_bounds__(kThreads) void select_lds_kernel(SelectArgs p) {
+  extern __shared__ float row[];
+  __shared__ int slots[2][kWaves];
+  __shared__ int scan_lds[kWaves];
+  __shared__ float max_lds[kWaves];
+  const int tid = threadIdx.x;
+  const int Tn = p.NB * p.BS;
+  uint32_t* keys = (uint32_t*)(row + Tn);
+  const int64_t r = blockIdx.x;
+  const int b = (int)((r / p.Hkv) % p.B);
+  const int64_t base = r * Tn;
+  const int32_t* trow = p.table + (int64_t)b * p.NB;
+
+  stage_row<T>(p.scores, base, Tn, row);
+  float rmax = 1.f;
+  if (p.red && p.norm_r) {
+    float m = -INFINITY;
+    for (int t = tid; t < Tn; t += kThreads) m = fmaxf(m, Elem<T>::ld(p.red, base + t));
+    rmax = block_max_of(m, max_lds);
+  } else {
+    __syncthreads();
+  }
+
+  const bool pooled = p.ksize > 1 && (p.continues || p.compressed[b] == 0);
+  const int half = p.ksize / 2;
+  for (int t = tid; t < Tn; t += kThreads) {
+    float v = row[t];
+    if (pooled) {
+      const int lo = max(t - half, 0), hi = min(t + half, Tn - 1);
+      if (p.mode == ZP_POOL_MAX) {
+        v = row[lo];
+        for (int i = lo + 1; i <= hi; ++i) v = fmaxf(v, row[i]);
+      } else {
+        float acc = 0.f;
+        for (int i = lo; i <= hi; ++i) acc += row[i];
+        v = Elem<T>::rnd(acc / (float)p.ksize);
+      }
+    }
+    const int j = t / p.BS, slot = t - j * p.BS;
+    v = select_finish<T>(p, v, t, base, trow[j], slot, rmax);
+    keys[t] = score_key(v, p.low_bit);
+  }
+  __syncthreads();
+
+  const int chunk = (Tn + kThreads - 1) / kThreads;
+  const int s0 = min(tid * chunk, Tn), s1 = min(s0 + chunk, Tn);
+  uint32_t prefix = 0;
+  int pp = 0;
+  for (int bit = 31; bit >= p.low_bit; --bit) {
+    const uint32_t cand = prefix | (1u << bit);
+    int c = 0;
+    for (int s = s0; s < s1; ++s) c += keys[s] >= cand ? 1 : 0;
+    if (block_count(c, slots[pp]) >= p.k) prefix = cand;
+    pp ^= 1;
+  }
+  int cg = 0, ce = 0;
+  for (int s = s0; s < s1; ++s) {
+    cg += keys[s] > prefix ? 1 : 0;
+    ce += keys[s] == prefix ? 1 : 0;
+  }
+  const int need_eq = p.k - block_count(cg, slots[pp]);
+  int inc = ce;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    int t = __shfl_up(inc, o, 64);
+    if (lane_id() >= o) inc += t;
+  }
+  if (lane_id() == 63) scan_lds[wave_id()] = inc;
+  __syncthreads();
+  int rank = inc - ce;
+  for (int i = 0; i < wave_id(); ++i) rank += scan_lds[i];
+  uint8_t* fl = (uint8_t*)row;
+  for (int s = s0; s < s1; ++s) {
+    const uint32_t key = keys[s];
+    uint8_t f = key > prefix ? 1 : 0;
+    if (key == prefix) { f = rank < need_eq ? 1 : 0; ++rank; }
+    fl[s] = f;
+  }
+  __syncthreads();
+  write_flags(fl, p.flag, base, Tn);
+}
+
 }  // namespace
 
 extern "C" int zp_topk_mask(const void* scores, uint8_t* flag_out, int32_t rows, int32_t Tn,
@@ -113,6 +395,58 @@ extern "C" int zp_topk_mask(const void* scores, uint8_t* flag_out, int32_t rows,
   } while (0)
   ZP_DISPATCH_DTYPE(dtype, ZP_TOPK_LAUNCH());
 #undef ZP_TOPK_LAUNCH
+  ZP_LAUNCH_CHECK();
+  return ZP_OK;
+}
+
+extern "C" int zp_select_topk(const void* scores, void* scores_out, const void* redundancy,
+                              uint8_t* flag_out, const int32_t* block_table,
+                              const uint8_t* compressed, int32_t L, int32_t B, int32_t NB,
+                              int32_t BS, int32_t Hkv, int32_t pool_kernel_size,
+                              int32_t continues_pooling, int32_t pool_mode, int32_t max_norm_red,
+                              double redudancy_lambda, int32_t sink_len, int32_t window,
+                              int32_t mask_pad, int32_t k, int32_t dtype, void* stream) {
+  ZP_REQUIRE(L >= 0 && B >= 0 && NB > 0 && BS > 0 && Hkv > 0, "select_topk: bad dims");
+  const int64_t Tn = (int64_t)NB * BS;
+  ZP_REQUIRE(k >= 0 && k <= Tn, "select_topk: k=%d out of range for a row of %lld", k, (long long)Tn);
+  ZP_REQUIRE(pool_kernel_size <= 1 || (pool_kernel_size & 1),
+             "select_topk: pooling kernel_size %d must be odd", pool_kernel_size);
+  ZP_REQUIRE(pool_mode == ZP_POOL_MAX || pool_mode == ZP_POOL_AVG, "select_topk: unknown pooling mode %d",
+             pool_mode);
+  ZP_REQUIRE(window >= 0 && window <= BS, "select_topk: window %d outside [0, BS=%d]", window, BS);
+  ZP_REQUIRE(sink_len >= 0, "select_topk: negative sink_len");
+  ZP_REQUIRE(dtype >= ZP_BF16 && dtype <= ZP_F32, "select_topk: unknown dtype tag %d", dtype);
+  ZP_REQUIRE(Tn * 8 <= 150 * 1024, "select_topk: row of %lld tokens exceeds LDS", (long long)Tn);
+  if (L == 0 || B == 0) return ZP_OK;
+  ZP_REQUIRE(scores && flag_out && block_table && compressed, "select_topk: null pointer");
+  hipStream_t st = (hipStream_t)stream;
+  SelectArgs p;
+  p.scores = scores; p.scores_out = scores_out; p.red = redundancy; p.flag = flag_out;
+  p.table = block_table; p.compressed = compressed;
+  p.B = B; p.NB = NB; p.BS = BS; p.Hkv = Hkv; p.ksize = pool_kernel_size;
+  p.continues = continues_pooling; p.mode = pool_mode; p.norm_r = max_norm_red;
+  p.lam = (float)redudancy_lambda; p.one_minus_lam = (float)(1.0 - redudancy_lambda);
+  p.sink_len = sink_len; p.window = window; p.mask_pad = mask_pad; p.k = k;
+  p.low_bit = dtype == ZP_BF16 ? 16 : (dtype == ZP_F16 ? 13 : 0);
+  dim3 grid((unsigned)((int64_t)L * B * Hkv));
+  const bool in_regs = Tn <= 10 * kThreads && pool_kernel_size <= 2 * kSelHalf + 1;
+  const size_t smem = (size_t)Tn * (in_regs ? 4 : 8);
+#define ZP_SELECT_LAUNCH(KERNEL)                                                                  \
+  do {                                                                                            \
+    if (smem > 64 * 1024 &&                                                                       \
+        hipFuncSetAttribute((const void*)KERNEL, hipFuncAttributeMaxDynamicSharedMemorySize,      \
+                            (int)smem) != hipSuccess) {                                           \
+      zp_set_error("select_topk: cannot reserve %zu bytes of LDS", smem);                         \
+      return ZP_EHIP;                                                                             \
+    }                                                                                             \
+    hipLaunchKernelGGL(KERNEL, grid, dim3(kThreads), smem, st, p);                                \
+  } while (0)
+  if (in_regs) {
+    ZP_DISPATCH_DTYPE(dtype, ZP_SELECT_LAUNCH((select_reg_kernel<T, 10>)));
+  } else {
+    ZP_DISPATCH_DTYPE(dtype, ZP_SELECT_LAUNCH((select_lds_kernel<T>)));
+  }
+#undef ZP_SELECT_LAUNCH
   ZP_LAUNCH_CHECK();
   return ZP_OK;
 }

@@ -11,9 +11,10 @@ from zipage_amd.kernel.utils import topk_mask
 from zipage_amd.kernel.compress_kv import compress_kv
 from zipage_amd.kernel.compress_score import compress_score
 from zipage_amd.kernel.pooling import pool_scores
+from zipage_amd.kernel.select import select_topk
 
 __all__ = [
     "store_query_cache", "attention_score", "global_score", "window_mask", "score_epilogue",
     "key_norm", "lightning_redudancy_score", "raw_redudancy_score", "topk_mask", "compress_kv",
-    "compress_score", "pool_scores",
+    "compress_score", "pool_scores", "select_topk",
 ]
