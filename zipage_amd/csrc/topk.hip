@@ -187,21 +187,24 @@ __global__ __launch_bounds__(kThreads) void select_reg_kernel(SelectArgs p) {
   const int64_t r = blockIdx.x;
   const int b = (int)((r / p.Hkv) % p.B);
   const int64_t base = r * Tn;
-  const int32_t* trow = p.table + (int64_t)b * p.NB;
+  int* trow = (int*)(row + Tn);  // the sequence's page codes, NB words behind the row
 
+  // every global read of the prologue is issued before the first wait
+  const uint8_t was_compressed = p.compressed[b];
+  for (int i = tid; i < p.NB; i += kThreads) trow[i] = p.table[(int64_t)b * p.NB + i];
   stage_row<T>(p.scores, base, Tn, row);
   float rmax = 1.f;
   if (p.red && p.norm_r) {
     float m = -INFINITY;
     for (int t = tid; t < Tn; t += kThreads) m = fmaxf(m, Elem<T>::ld(p.red, base + t));
-    rmax = block_max_of(m, max_lds);  // its barrier also publishes row[]
+    rmax = block_max_of(m, max_lds);  // its barrier also publishes row[] and trow[]
   } else {
     __syncthreads();
   }
 
   const int chunk = (Tn + kThreads - 1) / kThreads;  // <= PER
   const int s0 = min(tid * chunk, Tn), s1 = min(s0 + chunk, Tn);
-  const bool pooled = p.ksize > 1 && (p.continues || p.compressed[b] == 0);
+  const bool pooled = p.ksize > 1 && (p.continues || was_compressed == 0);
   const int half = pooled ? p.ksize / 2 : 0;
   const bool is_max = p.mode == ZP_POOL_MAX;
   float win[PER + 2 * kSelHalf];
@@ -430,7 +433,7 @@ extern "C" int zp_select_topk(const void* scores, void* scores_out, const void* 
   p.low_bit = dtype == ZP_BF16 ? 16 : (dtype == ZP_F16 ? 13 : 0);
   dim3 grid((unsigned)((int64_t)L * B * Hkv));
   const bool in_regs = Tn <= 10 * kThreads && pool_kernel_size <= 2 * kSelHalf + 1;
-  const size_t smem = (size_t)Tn * (in_regs ? 4 : 8);
+  const size_t smem = in_regs ? (size_t)Tn * 4 + (size_t)NB * 4 : (size_t)Tn * 8;
 #define ZP_SELECT_LAUNCH(KERNEL)                                                                  \
   do {                                                                                            \
     if (smem > 64 * 1024 &&                                                                       \
