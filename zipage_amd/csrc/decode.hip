@@ -78,7 +78,9 @@ struct DecodeArgs {
 
 // K and V rows are read exactly once per step: non-temporal loads stream them past L2
 // (measured 5.7 -> 6.3 TB/s at 256 sequences x 2176 tokens).
+#ifndef ZP_DEC_LOAD
 #define ZP_DEC_LOAD(ptr) __builtin_nontemporal_load(ptr)
+#endif
 constexpr int kMaxTablePages = 256;     // block-table entries per sequence (the LDS logits cap the context first)
 constexpr int kGroups = kThreads / 8;  // token rows in flight per step of the workgroup
 constexpr int kUnroll = 4;             // rows per lane group and loop trip (must be even)

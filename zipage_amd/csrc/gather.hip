@@ -62,9 +62,14 @@ struct CompactArgs {
 };
 
 // Survivors are written once and not read again by this kernel: non-temporal stores keep them
-// from displacing the gather's source lines in L2 (measured at 256 sequences: 5.1 -> 6.0 TB/s).
+// from displacing the gather's source lines in L2 (measured at 256 sequences on one allocation:
+// 704 -> 686 us per launch; non-temporal loads on top: 720 us).
+#ifndef ZP_NT_LOAD
 #define ZP_NT_LOAD(ptr) (*(ptr))
+#endif
+#ifndef ZP_NT_STORE
 #define ZP_NT_STORE(v, ptr) __builtin_nontemporal_store(v, ptr)
+#endif
 // POW2: page size and pieces-per-vector are powers of two, so every index split is a shift.
 template <typename P, int R, bool HAS_B, bool POW2>
 __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
