@@ -129,8 +129,8 @@ def end_to_end(requests=256, prompt=512, out_tokens=4096, async_compress=True, r
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--config", type=int, default=2, choices=[2, 4, 5],
                     help="workload, numbered from 1 as in BASELINE.json: 2 = 64 ragged sequences, one "
@@ -219,18 +219,25 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
-    timer = StageTimer(True)
+    # timed region: only the roofline kernel carries events (each event pair costs the stream a
+    # few microseconds, 8 % of a step when every stage has one)
+    kv_timer = StageTimer(True, only=("compress_kv",))
     t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(kv_timer)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    # the per-stage breakdown comes from a second, untimed pass with events around every stage
+    timer = StageTimer(True)
     for _ in range(args.steps):
         step(timer)
     torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
 
     stage_s = timer.seconds()
     ms_per_step = elapsed / args.steps * 1e3
     seqs_per_s = wl.B / (elapsed / args.steps)
     alg = algorithmic_bytes(wl, cfg)  # one layer
-    kv_s = stage_s["compress_kv"] / (args.steps * layers)
+    kv_s = kv_timer.seconds()["compress_kv"] / (args.steps * layers)
     achieved = alg["compress_kv"] / kv_s / 1e9
     stages_ms = {k: round(v / (args.steps * layers) * 1e3, 4) for k, v in stage_s.items()}
     gpu_ms = sum(stage_s.values()) / (args.steps * layers) * 1e3  # per layer

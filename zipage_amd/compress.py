@@ -58,12 +58,13 @@ class CompressConfig:
 class StageTimer:
     """Optional per-stage device timing with the reference's stage names."""
 
-    def __init__(self, enabled: bool):
+    def __init__(self, enabled: bool, only: tuple[str, ...] | None = None):
         self.enabled = enabled
+        self.only = only      # time just these stages (every event pair costs a few microseconds)
         self.spans = []
 
     def start(self, name):
-        if not self.enabled:
+        if not self.enabled or (self.only is not None and name not in self.only):
             return None
         st, ed = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         st.record()
