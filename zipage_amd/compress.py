@@ -1,8 +1,11 @@
-"""One layer chunk of the compression pipeline on the GPU, in the reference's stage order.
+"""One layer chunk of the compression pipeline on the GPU.
 
 Host-side mirror of the body of ``ModelRunner.compress``
 (zipage/engine/model_runner.py:466-622): the same stages with the same switches, each
-dispatched to its HIP entry point.  Nothing here synchronises with the host: the
+dispatched to its HIP entry point.  The redundancy score only reads the key cache, so it is
+launched before the selection stages, which then run as one launch (pooling, combine, sink /
+window / pad masks, top-k); ``fused_select=False`` keeps them as the reference's separate
+stages, in its order.  Nothing here synchronises with the host: the
 reference's ``torch.all(compressed)`` test before pooling (model_runner.py:501) only skips
 work whose result equals its input, so pooling is decided per sequence on the device.
 """
