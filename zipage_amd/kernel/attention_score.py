@@ -38,6 +38,8 @@ def attention_score(k_cache: torch.Tensor, query_cache: torch.Tensor, seq_idx: t
     logits = None
     if return_logits:
         logits = torch.full((L, B, Hq, W, NB * BS), -float("inf"), device=dev, dtype=dt)
+    if L == 0 or B == 0:  # nothing to score: empty outputs, as the torch ops would give
+        return (scores, logits) if return_logits else scores
     lib = _lib.load()
     ws_bytes = lib.zp_attention_score_workspace(L, B, NB, BS, Hkv, Hq, W)
     ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8) if ws_bytes else None

@@ -20,6 +20,8 @@ def compress_kv(key: torch.Tensor, value: torch.Tensor, flag: torch.Tensor,
     assert block_table.shape == (B, NB) and block_table.is_contiguous()
     assert target_block_table.shape[0] == B and target_block_table.is_contiguous()
     assert block_table.dtype == torch.int32 and target_block_table.dtype == torch.int32
+    if flag.numel() == 0:
+        return None
     _lib.call("zp_compress_kv", _lib.dev_ptr(key), _lib.dev_ptr(value), _lib.dev_ptr(flag),
               _lib.dev_ptr(block_table), _lib.dev_ptr(target_block_table), L, B, NB, BS, Hkv, D,
               num_pages, target_block_table.shape[1],

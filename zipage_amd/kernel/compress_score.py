@@ -16,6 +16,8 @@ def compress_score(score_cache: torch.Tensor, flag: torch.Tensor, block_table: t
     assert block_table.shape == (B, NB) and block_table.is_contiguous()
     assert target_block_table.shape[0] == B and target_block_table.is_contiguous()
     assert block_table.dtype == torch.int32 and target_block_table.dtype == torch.int32
+    if flag.numel() == 0:
+        return score_cache
     _lib.call("zp_compress_score", _lib.dev_ptr(score_cache), _lib.dev_ptr(flag),
               _lib.dev_ptr(block_table), _lib.dev_ptr(target_block_table), L, B, NB, BS, Hkv,
               score_cache.shape[1], target_block_table.shape[1], score_cache.stride(0),

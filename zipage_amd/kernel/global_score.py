@@ -25,6 +25,8 @@ def global_score(reduced_scores: torch.Tensor, score_cache: torch.Tensor,
     assert reduced_scores.dtype == score_cache.dtype
     assert block_table.dtype == torch.int32 and compressed.dtype == torch.bool
     compressed = compressed.contiguous()
+    if reduced_scores.numel() == 0:
+        return reduced_scores
     _lib.call("zp_global_score", _lib.dev_ptr(reduced_scores), _lib.dev_ptr(score_cache),
               _lib.dev_ptr(block_table), _lib.dev_ptr(compressed), L, B, NB, BS, Hkv, num_pages,
               score_cache.stride(0), score_cache.stride(1), float(decay_factor),

@@ -21,6 +21,8 @@ def key_norm(key_cache: torch.Tensor, block_table: torch.Tensor, norm_epsilon: f
     B, NB = block_table.shape
     assert block_table.is_contiguous() and block_table.dtype == torch.int32
     out = torch.empty((L, B, Hkv, NB, BS), device=key_cache.device, dtype=key_cache.dtype)
+    if out.numel() == 0:
+        return out
     _lib.call("zp_key_norm", _lib.dev_ptr(key_cache), _lib.dev_ptr(block_table), _lib.dev_ptr(out),
               L, B, NB, BS, Hkv, D, num_pages, key_cache.stride(0), key_cache.stride(1),
               float(norm_epsilon), _lib.dtype_tag(key_cache), _lib.stream_ptr(key_cache))

@@ -21,6 +21,8 @@ def lightning_redudancy_score(key_cache: torch.Tensor, block_table: torch.Tensor
     dev, dt = key_cache.device, key_cache.dtype
     red = torch.empty((L, B, Hkv, NB, BS), device=dev, dtype=dt)
     logits = torch.empty_like(red) if return_logits else None
+    if red.numel() == 0:
+        return (logits, red) if return_logits else red
     _lib.call("zp_redundancy_lightning", _lib.dev_ptr(key_cache), _lib.dev_ptr(block_table),
               _lib.dev_ptr(red), _lib.dev_ptr(logits), L, B, NB, BS, Hkv, D, num_pages,
               key_cache.stride(0), key_cache.stride(1), float(threshold), float(temperature),

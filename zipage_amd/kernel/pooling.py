@@ -17,6 +17,8 @@ def pool_scores(scores: torch.Tensor, compressed: torch.Tensor, kernel_size: int
     L, B, Hkv, NB, BS = scores.shape
     assert scores.is_contiguous() and compressed.dtype == torch.bool
     out = torch.empty_like(scores)
+    if out.numel() == 0:
+        return out
     _lib.call("zp_pool_scores", _lib.dev_ptr(scores), _lib.dev_ptr(out),
               _lib.dev_ptr(compressed.contiguous()), L, B, Hkv, NB * BS, int(kernel_size),
               int(continues_pooling), _MODES[mode], _lib.dtype_tag(scores),

@@ -20,6 +20,8 @@ def raw_redudancy_score(key_cache: torch.Tensor, block_table: torch.Tensor,
     dev, dt = key_cache.device, key_cache.dtype
     red = torch.empty((L, B, Hkv, NB, BS), device=dev, dtype=dt)
     logits = torch.empty((L, B, Hkv, NB * BS), device=dev, dtype=dt) if return_logits else None
+    if red.numel() == 0:
+        return (logits, red) if return_logits else red
     lib = _lib.load()
     ws_bytes = lib.zp_redundancy_raw_workspace(L, B, NB, BS, Hkv)
     ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8) if ws_bytes else None

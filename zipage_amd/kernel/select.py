@@ -29,6 +29,8 @@ def select_topk(scores: torch.Tensor, block_table: torch.Tensor, compressed: tor
         raise RuntimeError(f"selected index k out of range: k={k}, row length {NB * BS}")
     flag = torch.empty(scores.shape, device=scores.device, dtype=torch.bool)
     out = torch.empty_like(scores) if return_scores else None
+    if flag.numel() == 0:
+        return (flag, out) if return_scores else flag
     _lib.call("zp_select_topk", _lib.dev_ptr(scores), _lib.dev_ptr(out), _lib.dev_ptr(redundancy),
               _lib.dev_ptr(flag), _lib.dev_ptr(block_table), _lib.dev_ptr(compressed.contiguous()),
               L, B, NB, BS, Hkv, int(pooling_size), int(continues_pooling), _MODES[pooling_mode],

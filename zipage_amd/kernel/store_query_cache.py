@@ -15,7 +15,7 @@ def store_query_cache(query: torch.Tensor, query_cache: torch.Tensor, slot_mappi
     N = slot_mapping.shape[0]
     _, num_heads, head_dim = query.shape
     D = num_heads * head_dim
-    if query_cache.numel() == 0:  # warmup
+    if query_cache.numel() == 0 or N == 0:  # warmup, or nothing to store
         return
     assert query.stride(-1) == 1
     assert query.stride(1) == head_dim

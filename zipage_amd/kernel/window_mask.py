@@ -15,6 +15,8 @@ def score_epilogue(scores, block_table, redundancy=None, *, max_norm_scores=Fals
     if redundancy is not None:
         assert redundancy.shape == scores.shape and redundancy.dtype == scores.dtype
         assert redundancy.is_contiguous()
+    if scores.numel() == 0:
+        return scores
     _lib.call("zp_score_epilogue", _lib.dev_ptr(scores), _lib.dev_ptr(redundancy),
               _lib.dev_ptr(block_table), L, B, NB, BS, Hkv, int(max_norm_scores),
               int(max_norm_red), float(redudancy_lambda), int(sink_len), int(window),
