@@ -330,8 +330,13 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
             }
             if constexpr (PASS == 0) {
               // max of sign(scale)*acc; scaling is monotone, so it is applied once at the end
+              if (sgn > 0.f) {  // block-uniform: the negation is a free source modifier
 #pragma unroll
-              for (int r = 0; r < 16; ++r) run[r] = fmaxf(run[r], sgn * acc[r]);
+                for (int r = 0; r < 16; ++r) run[r] = fmaxf(run[r], acc[r]);
+              } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) run[r] = fmaxf(run[r], -acc[r]);
+              }
               if constexpr (LOGITS) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
@@ -358,8 +363,10 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
                   run[r] += e0;
                   run[r + 1] += e1;
                 } else {
+                  // rounding to the cache dtype is monotone, so max over the group of the rounded
+                  // probabilities == rounded max: groups of >= 2 rows round after their maximum
                   float p0 = e0 * invl[r], p1 = e1 * invl[r + 1];
-                  Rnd<T>::pair(p0, p1);
+                  if (p.Gp < 2) Rnd<T>::pair(p0, p1);
                   pv[r] = p0;
                   pv[r + 1] = p1;
                 }
@@ -377,11 +384,21 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
 #pragma unroll
                     for (int q = 0; q < 4; ++q) q4[q] = fmaxf(q4[q], lane_xor32(q4[q]));
                   }
+                  if (Gp < 16) {
+                    Rnd<T>::pair(q4[0], q4[1]);
+                    Rnd<T>::pair(q4[2], q4[3]);
+                  }
                   if (Gp >= 16) {
                     q4[0] = fmaxf(q4[0], q4[1]);
                     q4[2] = fmaxf(q4[2], q4[3]);
-                    if (Gp >= 32) red = fmaxf(q4[0], q4[2]);
-                    else red = p.reduce_max ? fmaxf(q4[0], q4[2]) : q4[0] + q4[2];
+                    if (Gp >= 32) {
+                      red = fmaxf(q4[0], q4[2]);
+                      float dummy = red;
+                      Rnd<T>::pair(red, dummy);
+                    } else {
+                      Rnd<T>::pair(q4[0], q4[2]);
+                      red = p.reduce_max ? fmaxf(q4[0], q4[2]) : q4[0] + q4[2];
+                    }
                   } else {
                     red = p.reduce_max ? fmaxf(fmaxf(q4[0], q4[1]), fmaxf(q4[2], q4[3]))
                                        : (q4[0] + q4[1]) + (q4[2] + q4[3]);
@@ -391,6 +408,8 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
                   if (Gp == 2) {
 #pragma unroll
                     for (int q = 0; q < 8; ++q) t8[q] = fmaxf(pv[2 * q], pv[2 * q + 1]);
+#pragma unroll
+                    for (int q = 0; q < 8; q += 2) Rnd<T>::pair(t8[q], t8[q + 1]);
                   } else {
 #pragma unroll
                     for (int q = 0; q < 8; ++q)
