@@ -127,3 +127,30 @@ def test_select_topk_rejects_bad_arguments(dev):
         select_topk(scores, enc, comp, 256, pooling_size=4)
     with pytest.raises(RuntimeError, match="window"):
         select_topk(scores, enc, comp, 256, window=257)
+
+
+def test_select_topk_random_shapes(dev):
+    """Thirty random small shapes (rows shorter than the workgroup, pages of 8 to 64 slots, chunk
+    boundaries that split pages, k anywhere in [0, T]) against the oracle's separate stages."""
+    from zipage_amd.kernel import select_topk
+    g = torch.Generator().manual_seed(71)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    for trial in range(30):
+        dtype = [torch.float32, torch.bfloat16, torch.float16][trial % 3]
+        L, B, Hkv = ri(1, 2), ri(1, 3), ri(1, 3)
+        BS, NB = [8, 16, 24, 32, 64][ri(0, 4)], ri(1, 12)
+        enc = _tables(B, NB, 100 + trial)
+        scores = (torch.randint(0, 30, (L, B, Hkv, NB, BS), generator=g).float() / 64.0).to(dtype)
+        compressed = torch.rand(B, generator=g) < 0.5
+        pool = [0, 3, 5, 7, 9][ri(0, 4)]
+        k = ri(0, NB * BS)
+        window, sink = ri(0, BS), ri(0, 5)
+        want_flag, want_scores = _oracle(scores, enc, compressed, k, pool, bool(trial & 1), "max",
+                                         None, False, 0.0, sink, window)
+        flag, out = select_topk(scores.to(dev), enc.to(dev), compressed.to(dev), k,
+                                pooling_size=pool, continues_pooling=bool(trial & 1), sink_len=sink,
+                                window=window, mask_pad=True, return_scores=True)
+        case = dict(trial=trial, dtype=dtype, shape=(L, B, Hkv, NB, BS), pool=pool, k=k,
+                    window=window, sink=sink)
+        assert torch.equal(out.cpu(), want_scores), case
+        assert torch.equal(flag.cpu(), want_flag), case
