@@ -151,17 +151,4 @@ __device__ __forceinline__ uint64_t lanemask_lt() {
   return (1ull << lane_id()) - 1ull;
 }
 
-// Workgroups are dealt round-robin to the 8 XCDs (id % 8).  Work items whose low index bits
-// select a fixed byte lane of every cache row (one kv head = one 256-byte slice of each 2 KB
-// token row) would otherwise pin each XCD to a fraction of its L2 channels.  This remap gives
-// XCD x the contiguous item range [x*chunk, (x+1)*chunk), so neighbouring items (all heads of
-// one sequence) share an XCD and its L2.  Launch 8*chunk workgroups, chunk = ceil(n/8);
-// items >= n exit.
-constexpr int ZP_XCDS = 8;
-static inline unsigned zp_xcd_grid(int64_t n) { return (unsigned)(((n + ZP_XCDS - 1) / ZP_XCDS) * ZP_XCDS); }
-__device__ __forceinline__ int zp_xcd_item(int n) {
-  const int chunk = (n + ZP_XCDS - 1) / ZP_XCDS;
-  return (int)(blockIdx.x % ZP_XCDS) * chunk + (int)(blockIdx.x / ZP_XCDS);
-}
-
 struct __attribute__((aligned(16))) vec16 { uint32_t x, y, z, w; };
