@@ -122,6 +122,20 @@ template <> struct Rnd<F16> {
   }
 };
 
+// One v_max_f32, nothing else: fmaxf() makes the compiler quiet possible signalling NaNs first
+// (an extra v_max x,x per operand that is not known to be canonical, e.g. anything unpacked from
+// bf16 bits), which doubles or triples the cost of the max-heavy epilogues.  No NaN occurs here.
+__device__ __forceinline__ float vmax(float a, float b) {
+  float d;
+  asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+}
+__device__ __forceinline__ float vmax_neg(float a, float b) {  // max(a, -b)
+  float d;
+  asm("v_max_f32 %0, %1, -%2" : "=v"(d) : "v"(a), "v"(b));
+  return d;
+}
+
 // exp of a non-positive argument, natural base, via the hardware base-2 exponential.
 __device__ __forceinline__ float exp_neg(float x) {
 #ifdef ZP_DBG_NOEXP
@@ -130,9 +144,16 @@ __device__ __forceinline__ float exp_neg(float x) {
   return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
 }
 
-template <typename T, bool LOGITS>
+// GPC: padded GQA group size known at compile time (0: read it from the arguments); RMAXC: window
+// reduction known at compile time (0 mean, 1 max, -1: from the arguments).  The common shape
+// (group 4, mean) gets its own instantiation: straight-line epilogues instead of uniform branches
+// and compute-both-then-select.
+template <typename T, bool LOGITS, int GPC, int RMAXC>
 __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_OCC : 1)) void score_kernel(ScoreArgs p) {
   typedef Mma<T> M;
+  const int GpV = GPC > 0 ? GPC : p.Gp;
+  const int gsV = GPC == 8 ? 3 : GPC == 4 ? 2 : GPC == 2 ? 1 : p.gs;
+  const bool rmaxV = RMAXC >= 0 ? (RMAXC != 0) : (p.reduce_max != 0);
   typedef typename M::Frag Frag;
   constexpr int TN = M::TN, ROWB = M::ROWB, KS = M::KS;
   const int RW = p.RW, TW = kWaves / RW;  // row waves x token waves
@@ -235,7 +256,7 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
     // ---- A fragments: query rows of this wave's row block
     Frag afrag[KS];
     const int mrow = rb * 32 + col;                 // row this lane loads
-    const int a_w = mrow >> p.gs, a_g = mrow & (p.Gp - 1);
+    const int a_w = mrow >> gsV, a_g = mrow & (GpV - 1);
     const bool a_ok = active && seq_ok && a_w < p.W && a_g < p.G;
     {
       const char* qrow = p.q + ((int64_t)l * p.q_sl + (int64_t)seq * p.q_ss +
@@ -266,15 +287,15 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
           float v = pt[tid];
 #pragma unroll
           for (int w2 = 1; w2 < RW; ++w2)
-            v = p.reduce_max ? fmaxf(v, pt[w2 * TN + tid]) : v + pt[w2 * TN + tid];
+            v = rmaxV ? fmaxf(v, pt[w2 * TN + tid]) : v + pt[w2 * TN + tid];
           const int64_t oi = orow * Tn + (int64_t)j * p.BS + toff + tid;
           if (NR > 1) {
             float* wsp = p.ws + oi;
-            if (rr > 0) v = p.reduce_max ? fmaxf(v, *wsp) : v + *wsp;
+            if (rr > 0) v = rmaxV ? fmaxf(v, *wsp) : v + *wsp;
             if (rr + 1 < NR) *wsp = v;
           }
           if (rr + 1 == NR)
-            Elem<T>::st(p.out, oi, p.reduce_max ? v : Elem<T>::rnd(v / (float)p.W));
+            Elem<T>::st(p.out, oi, rmaxV ? v : Elem<T>::rnd(v / (float)p.W));
         }
       };
       float run[16];
@@ -324,7 +345,7 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
             if (last && (toff + st * 32 + 31 > p.BS - p.W)) {
 #pragma unroll
               for (int r = 0; r < 16; ++r) {
-                const int w = (row0 + (r >> 2) * 8 + (r & 3)) >> p.gs;
+                const int w = (row0 + (r >> 2) * 8 + (r & 3)) >> gsV;
                 if (slot > p.BS - p.W + w) acc[r] = -sgn * INFINITY;
               }
             }
@@ -332,16 +353,16 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
               // max of sign(scale)*acc; scaling is monotone, so it is applied once at the end
               if (sgn > 0.f) {  // block-uniform: the negation is a free source modifier
 #pragma unroll
-                for (int r = 0; r < 16; ++r) run[r] = fmaxf(run[r], acc[r]);
+                for (int r = 0; r < 16; ++r) run[r] = vmax(run[r], acc[r]);
               } else {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) run[r] = fmaxf(run[r], -acc[r]);
+                for (int r = 0; r < 16; ++r) run[r] = vmax_neg(run[r], acc[r]);
               }
               if constexpr (LOGITS) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                   const int m = row0 + (r >> 2) * 8 + (r & 3);
-                  const int w = m >> p.gs, g = m & (p.Gp - 1);
+                  const int w = m >> gsV, g = m & (GpV - 1);
                   if (w < p.W && g < p.G) {
                     const int64_t li =
                         ((((int64_t)l * p.B + b) * p.Hq + (int64_t)h * p.G + g) * p.W + w) * Tn +
@@ -365,66 +386,68 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
                 } else {
                   // rounding to the cache dtype is monotone, so max over the group of the rounded
                   // probabilities == rounded max: groups of >= 2 rows round after their maximum
-                  float p0 = e0 * invl[r], p1 = e1 * invl[r + 1];
-                  if (p.Gp < 2) Rnd<T>::pair(p0, p1);
-                  pv[r] = p0;
-                  pv[r + 1] = p1;
+                  pv[r] = e0 * invl[r];
+                  pv[r + 1] = e1 * invl[r + 1];
                 }
               }
               if constexpr (PASS == 2) {
                 // group max inside the lane, then window sum / max
                 float red;
-                const int Gp = p.Gp;
+                const int Gp = GpV;
+                if (Gp < 2) {  // no group: every probability is rounded on its own
+#pragma unroll
+                  for (int r = 0; r < 16; r += 2) Rnd<T>::pair(pv[r], pv[r + 1]);
+                }
                 if (Gp >= 4) {
                   float q4[4];
 #pragma unroll
                   for (int q = 0; q < 4; ++q)
-                    q4[q] = fmaxf(fmaxf(pv[4 * q], pv[4 * q + 1]), fmaxf(pv[4 * q + 2], pv[4 * q + 3]));
+                    q4[q] = vmax(vmax(pv[4 * q], pv[4 * q + 1]), vmax(pv[4 * q + 2], pv[4 * q + 3]));
                   if (Gp >= 8) {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) q4[q] = fmaxf(q4[q], lane_xor32(q4[q]));
+                    for (int q = 0; q < 4; ++q) q4[q] = vmax(q4[q], lane_xor32(q4[q]));
                   }
                   if (Gp < 16) {
                     Rnd<T>::pair(q4[0], q4[1]);
                     Rnd<T>::pair(q4[2], q4[3]);
                   }
                   if (Gp >= 16) {
-                    q4[0] = fmaxf(q4[0], q4[1]);
-                    q4[2] = fmaxf(q4[2], q4[3]);
+                    q4[0] = vmax(q4[0], q4[1]);
+                    q4[2] = vmax(q4[2], q4[3]);
                     if (Gp >= 32) {
-                      red = fmaxf(q4[0], q4[2]);
+                      red = vmax(q4[0], q4[2]);
                       float dummy = red;
                       Rnd<T>::pair(red, dummy);
                     } else {
                       Rnd<T>::pair(q4[0], q4[2]);
-                      red = p.reduce_max ? fmaxf(q4[0], q4[2]) : q4[0] + q4[2];
+                      red = rmaxV ? vmax(q4[0], q4[2]) : q4[0] + q4[2];
                     }
                   } else {
-                    red = p.reduce_max ? fmaxf(fmaxf(q4[0], q4[1]), fmaxf(q4[2], q4[3]))
+                    red = rmaxV ? vmax(vmax(q4[0], q4[1]), vmax(q4[2], q4[3]))
                                        : (q4[0] + q4[1]) + (q4[2] + q4[3]);
                   }
                 } else {
                   float t8[8];
                   if (Gp == 2) {
 #pragma unroll
-                    for (int q = 0; q < 8; ++q) t8[q] = fmaxf(pv[2 * q], pv[2 * q + 1]);
+                    for (int q = 0; q < 8; ++q) t8[q] = vmax(pv[2 * q], pv[2 * q + 1]);
 #pragma unroll
                     for (int q = 0; q < 8; q += 2) Rnd<T>::pair(t8[q], t8[q + 1]);
                   } else {
 #pragma unroll
                     for (int q = 0; q < 8; ++q)
-                      t8[q] = p.reduce_max ? fmaxf(pv[2 * q], pv[2 * q + 1]) : pv[2 * q] + pv[2 * q + 1];
+                      t8[q] = rmaxV ? vmax(pv[2 * q], pv[2 * q + 1]) : pv[2 * q] + pv[2 * q + 1];
                   }
-                  if (p.reduce_max) {
-                    red = fmaxf(fmaxf(fmaxf(t8[0], t8[1]), fmaxf(t8[2], t8[3])),
-                                fmaxf(fmaxf(t8[4], t8[5]), fmaxf(t8[6], t8[7])));
+                  if (rmaxV) {
+                    red = vmax(vmax(vmax(t8[0], t8[1]), vmax(t8[2], t8[3])),
+                                vmax(vmax(t8[4], t8[5]), vmax(t8[6], t8[7])));
                   } else {
                     red = ((t8[0] + t8[1]) + (t8[2] + t8[3])) + ((t8[4] + t8[5]) + (t8[6] + t8[7]));
                   }
                 }
                 if (Gp < 8) {  // the two lane halves hold different windows
                   const float o = lane_xor32(red);
-                  red = p.reduce_max ? fmaxf(red, o) : red + o;
+                  red = rmaxV ? vmax(red, o) : red + o;
                 }
                 if (half == 0) part[((tile & 1) * kRowWaves + rbw) * TN + st * 32 + col] = red;
               }
@@ -464,7 +487,7 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
             mx[r] = Elem<T>::rnd(v * ascale);
           } else {
             const int m = row0 + (r >> 2) * 8 + (r & 3);
-            const bool ok = active && (m >> p.gs) < p.W && (m & (p.Gp - 1)) < p.G;
+            const bool ok = active && (m >> gsV) < p.W && (m & (GpV - 1)) < p.G;
             invl[r] = ok ? 1.f / v : 0.f;
           }
         }
@@ -560,15 +583,27 @@ extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
     const size_t smem = 2 * (size_t)Mma<T>::TN * Mma<T>::ROWB +                                  \
                         sizeof(float) * (2 * kRowWaves * Mma<T>::TN + kWaves * 32) + sizeof(int) * 2 * NB;            \
     if (smem > 64 * 1024 &&                                                                      \
-        (hipFuncSetAttribute((const void*)score_kernel<T, false>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+        (hipFuncSetAttribute((const void*)score_kernel<T, false, 0, -1>, hipFuncAttributeMaxDynamicSharedMemorySize, \
                             (int)smem) != hipSuccess ||                                         \
-         hipFuncSetAttribute((const void*)score_kernel<T, true>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+         hipFuncSetAttribute((const void*)score_kernel<T, false, 4, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                            (int)smem) != hipSuccess ||                                         \
+         hipFuncSetAttribute((const void*)score_kernel<T, false, 2, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                            (int)smem) != hipSuccess ||                                         \
+         hipFuncSetAttribute((const void*)score_kernel<T, false, 8, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                            (int)smem) != hipSuccess ||                                         \
+         hipFuncSetAttribute((const void*)score_kernel<T, true, 0, -1>, hipFuncAttributeMaxDynamicSharedMemorySize, \
                             (int)smem) != hipSuccess)) {                                          \
       zp_set_error("attention_score: cannot reserve %zu bytes of LDS", smem);                    \
       return ZP_EHIP;                                                                            \
     }                                                                                            \
-    if (logits_out) hipLaunchKernelGGL((score_kernel<T, true>), grid, dim3(kThreads), smem, st, a);  \
-    else hipLaunchKernelGGL((score_kernel<T, false>), grid, dim3(kThreads), smem, st, a);        \
+    if (logits_out) hipLaunchKernelGGL((score_kernel<T, true, 0, -1>), grid, dim3(kThreads), smem, st, a);  \
+    else if (T::bytes == 2 && Gp == 4 && !a.reduce_max)                                          \
+      hipLaunchKernelGGL((score_kernel<T, false, 4, 0>), grid, dim3(kThreads), smem, st, a);     \
+    else if (T::bytes == 2 && Gp == 2 && !a.reduce_max)                                          \
+      hipLaunchKernelGGL((score_kernel<T, false, 2, 0>), grid, dim3(kThreads), smem, st, a);     \
+    else if (T::bytes == 2 && Gp == 8 && !a.reduce_max)                                          \
+      hipLaunchKernelGGL((score_kernel<T, false, 8, 0>), grid, dim3(kThreads), smem, st, a);     \
+    else hipLaunchKernelGGL((score_kernel<T, false, 0, -1>), grid, dim3(kThreads), smem, st, a); \
   } while (0)
   ZP_DISPATCH_DTYPE(dtype, ZP_SCORE_LAUNCH());
 #undef ZP_SCORE_LAUNCH
