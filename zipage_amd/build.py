@@ -28,10 +28,7 @@ def sources():
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
-def build(verbose: bool = True) -> str:
-    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    extra = os.environ.get("ZP_EXTRA_HIPCC_FLAGS", "").split()
-    cmd = [hipcc, *FLAGS, *extra, *sources(), "-o", LIB + ".tmp"]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -41,6 +38,23 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{proc.stdout}\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+
+
+def build(verbose: bool = True, jobs: int | None = None) -> str:
+    """Compile every source to an object file (in parallel) and link the shared object."""
+    from concurrent.futures import ThreadPoolExecutor
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    extra = os.environ.get("ZP_EXTRA_HIPCC_FLAGS", "").split()
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    compile_flags = [f for f in FLAGS if f != "-shared"]
+    srcs = sources()
+    objs = [os.path.join(objdir, os.path.basename(s)[:-4] + ".o") for s in srcs]
+    jobs = jobs or min(len(srcs), os.cpu_count() or 1, 16)
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(lambda so: _run([hipcc, *compile_flags, *extra, "-c", so[0], "-o", so[1]], verbose),
+                      zip(srcs, objs)))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB + ".tmp"], verbose)
     os.replace(LIB + ".tmp", LIB)
     return LIB
 
