@@ -27,7 +27,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes one compaction launch moves per (sequence, layer), from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE scaled by a plain copy kernel (profiles/pipeline_cfg2_b64.md)
-COMPACT_TRAFFIC_PER_SEQ_LAYER = 16_802_753
+COMPACT_TRAFFIC_PER_SEQ_LAYER = 16_803_258
 
 
 def cpu_baseline(wl, cfg, sample_seqs, budget_s=30.0):
