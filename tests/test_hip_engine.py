@@ -213,3 +213,29 @@ def test_prefix_cache_shares_pages_between_equal_prompts(dev):
     assert out[1]["token_ids"][0] == ref[0]["token_ids"][0]
     pool = eng.scheduler.pool
     assert pool.num_free == cfg.num_kvcache_blocks and not pool.refcount.any()
+
+
+def test_reference_script_switches_through_the_engine(dev):
+    """The switch set of the reference's scripts (global score with decay 0.8 and max-norm,
+    lightning redundancy, pooling, attention sink) through the whole engine: the score cache is
+    carried and compacted with the K/V pages, every request completes with the compression count
+    its length dictates, graph replay and eager launches agree token for token, and all pages and
+    rows come back."""
+    from zipage_amd.compress import CompressConfig
+    sw = CompressConfig(use_global_score=True, decay_factor=0.8, max_norm=True, enable_pooling=True,
+                        pooling_size=5, use_redudancy=True, lightning_redudancy=True,
+                        use_attention_sink=True, sink_len=4)
+    prompts = _prompts(4, [120, 300, 640, 900], seed=3)
+    e1, a = _generate(_cfg(use_graph=False, compress=sw), prompts, 650)
+    e2, b = _generate(_cfg(use_graph=True, compress=sw), prompts, 650)
+    assert e1.runner.score_cache is not None and e1.stats["compress_calls"] > 2
+    BS, cap = 256, 3
+    for p, x, y in zip(prompts, a, b):
+        assert len(x["token_ids"]) == 650 and x["token_ids"] == y["token_ids"]
+        total = len(p) + 650
+        first = max(cap, -(-len(p) // BS)) * BS + 1
+        want = 0 if total - 1 < first else 1 + (total - 1 - first) // BS
+        assert x["num_compressions"] == y["num_compressions"] == want
+    for eng in (e1, e2):
+        pool = eng.scheduler.pool
+        assert pool.num_free == eng.cfg.num_kvcache_blocks and not pool.refcount.any()
