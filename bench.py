@@ -62,7 +62,8 @@ def cpu_baseline(wl, cfg, sample_seqs, budget_s=30.0):
                       f"after 1 warm-up ({med * 1e3:.0f} ms per run)"}
 
 
-def end_to_end(requests=256, prompt=512, out_tokens=4096, async_compress=True, ragged=False):
+def end_to_end(requests=256, prompt=512, out_tokens=4096, async_compress=True, ragged=False,
+               script_switches=False):
     """BASELINE configs[4]: offline decode of a random-init Qwen3-8B with the KV budget on.
     Returns decode tokens/s (decode steps only, first decode step to the last, device-complete),
     the share of that time the compression kernels were running, and the bandwidth of the
@@ -76,7 +77,9 @@ def end_to_end(requests=256, prompt=512, out_tokens=4096, async_compress=True, r
                        num_kvcache_blocks=requests * 9 + 64, query_cache_len=16,
                        max_model_len=prompt + out_tokens + 1, enable_async_compress=async_compress,
                        max_compress_blocks=requests * 16,
-                       compress=CompressConfig(enable_pooling=True, pooling_size=5))
+                       compress=(CompressConfig(use_global_score=True, decay_factor=0.8, enable_pooling=True,
+                                                pooling_size=5, use_redudancy=True, lightning_redudancy=True)
+                                 if script_switches else CompressConfig(enable_pooling=True, pooling_size=5)))
     eng = ZipageEngine(cfg)
     g = torch.Generator().manual_seed(0)
     if ragged:
@@ -108,7 +111,9 @@ def end_to_end(requests=256, prompt=512, out_tokens=4096, async_compress=True, r
     out = {
         "workload": (f"configs[4]: random-init Qwen3-8B bf16, {requests} requests, "
                      f"{'ragged ' if ragged else ''}{prompt}-token prompts, {out_tokens} greedy tokens "
-                     "each, budget 8 pages x 256 tokens, window 16, max-pool 5, compression "
+                     "each, budget 8 pages x 256 tokens, window 16, "
+                     + ("global score (decay 0.8) + lightning redundancy + max-pool 5" if script_switches
+                        else "max-pool 5") + ", compression "
                      + ("on a side stream" if async_compress else "in line with the decode steps")),
         "decode_tok_per_s": round(st["decode_tokens"] / st["decode_s"], 1),
         "ms_per_decode_step": round(st["decode_s"] / st["decode_steps"] * 1e3, 3),
@@ -145,6 +150,9 @@ def main():
     ap.add_argument("--sync-compress", action="store_true",
                     help="end-to-end leg: compress in line with the decode steps instead of on "
                          "the side stream")
+    ap.add_argument("--script-switches", action="store_true",
+                    help="end-to-end leg: compress with the switch set of the reference's scripts "
+                         "(global score, lightning redundancy, pooling) instead of pooling alone")
     ap.add_argument("--ragged-prompts", action="store_true",
                     help="end-to-end leg: prompt lengths uniform in [P/2, 3P/2] so sequences reach "
                          "their budget on different steps")
@@ -176,7 +184,7 @@ def main():
     torch.cuda.set_device(0)
     if args.config == 5:
         e2e = end_to_end(args.requests, args.prompt, args.out_tokens, not args.sync_compress,
-                         args.ragged_prompts)
+                         args.ragged_prompts, args.script_switches)
         print(json.dumps({
             "metric": "decode tokens/sec", "value": e2e["decode_tok_per_s"], "unit": "tokens/s",
             "n_gpus": 1, "steps": e2e["decode_steps"], "warmup": 0,
@@ -268,7 +276,8 @@ def main():
         del wl
         torch.cuda.empty_cache()
         out["end_to_end"] = end_to_end(args.requests, args.prompt, args.out_tokens,
-                                       not args.sync_compress, args.ragged_prompts)
+                                       not args.sync_compress, args.ragged_prompts,
+                                       args.script_switches)
     print(json.dumps(out))
 
 
