@@ -518,10 +518,28 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gram_split_kernel(Gr
 
 // ------------------------------------------------------------------ lightning, whole page in LDS
 // Per-page variant for 16-bit caches and pages of up to 256 keys: the page is normalised and
-// split once into LDS (hi and lo planes, 2 x 68 KB), after which eight waves each own a
-// 32-row block and run over all column blocks with no further staging or barriers.
+// split once into LDS (hi and lo planes, 2 x 68 KB).  The Gram matrix is symmetric, so every
+// unordered pair of 32-key blocks is multiplied once: wave a takes the blocks (a, a+d mod n)
+// for d = 0..n/2 (the pairs at distance n/2 go to the lower half of the waves), which is 5 or 4
+// tiles per wave for a 256-key page instead of 8.  A tile only feeds the claim rule (its
+// entries over the threshold update the last-column-over-threshold of the keys on BOTH of its
+// sides); the row sums do not need the matrix at all:
+//     sum_{j != i} e_i.e_j = e_i . (sum_j e_j - e_i)
+// is one fp32 dot product per key against the page's summed key, done while the raw keys are
+// still in registers.  The values of the (at most one per key) claimed entries are recomputed
+// afterwards from the two planes.
 constexpr int kPageThreads = 512;
+constexpr int kPageWaves = kPageThreads / 64;
 constexpr int kPageRows = 256;
+
+// Largest value over the 32 lanes of a wave half.
+__device__ __forceinline__ int half_max_i(int v) {
+  v = max(v, dpp_row_ror<8>(v));
+  v = max(v, dpp_row_ror<4>(v));
+  v = max(v, dpp_row_ror<2>(v));
+  v = max(v, dpp_row_ror<1>(v));
+  return max(v, lane_xor16(v));
+}
 
 template <typename T>
 __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
@@ -536,6 +554,7 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
   float* l_sum = (float*)(smem + 2 * PLANE);
   float* l_val = l_sum + kPageRows;
   int* l_col = (int*)(l_val + kPageRows);
+  float* l_part = (float*)(l_col + kPageRows);     // [waves][kDmax] partial key sums
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
@@ -558,19 +577,24 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
   const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
   const char* page = p.k + (l * p.k_sl + (int64_t)rpid * p.k_sp) * 2 + (int64_t)h * p.D * 2;
 
-  // ---- stage: normalise and split every key of the page
+  // ---- stage: normalise and split every key of the page, sum the normalised keys
   {
     const int piece = tid % PIECES, row0 = tid / PIECES;       // 32 rows per iteration
     constexpr int ROWS_PER_IT = kPageThreads / PIECES;
     constexpr int ITERS = kPageRows / ROWS_PER_IT;
     // all loads of the page are in flight before the first one is consumed
     u32x4 raw[ITERS];
+    float rn[ITERS];
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int row = it * ROWS_PER_IT + row0;
       raw[it] = *(const u32x4*)(page + (int64_t)(row < p.BS ? row : 0) * k_row +
                                 (piece < dpieces ? piece : 0) * 16);
     }
+    if (tid < kPageRows) l_col[tid] = -1;
+    float cs[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) cs[q] = 0.f;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int row = it * ROWS_PER_IT + row0;
@@ -584,36 +608,80 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
         for (int q = 0; q < 8; ++q) ss += e[q] * e[q];
       }
       ss = pieces_sum<PIECES>(ss);
-      const float rn = 1.f / fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
+      rn[it] = 1.f / fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
       bf16x8_t hi, lo;
 #pragma unroll
-      for (int q = 0; q < 8; ++q) e[q] = ok ? e[q] * rn : 0.f;
+      for (int q = 0; q < 8; ++q) {
+        e[q] = ok ? e[q] * rn[it] : 0.f;
+        cs[q] += e[q];
+      }
       split8(e, hi, lo);
       if (row < p.BS) {
         *(bf16x8_t*)(hi_pl + row * ROWH + piece * 16) = hi;
         *(bf16x8_t*)(lo_pl + row * ROWH + piece * 16) = lo;
       }
     }
+    // the four key rows a wave handles per iteration sit 16 lanes apart
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      cs[q] += lane_xor16(cs[q]);
+      cs[q] += lane_xor32(cs[q]);
+    }
+    if (lane < PIECES) {
+      float* dst = l_part + wave * kDmax + piece * 8;
+      *(float4*)dst = make_float4(cs[0], cs[1], cs[2], cs[3]);
+      *(float4*)(dst + 4) = make_float4(cs[4], cs[5], cs[6], cs[7]);
+    }
+    __syncthreads();
+    // summed key (fixed order over the waves), then every key's dot product with the rest
+    float sv[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) sv[q] = 0.f;
+#pragma unroll
+    for (int w = 0; w < kPageWaves; ++w) {
+      const float* src = l_part + w * kDmax + piece * 8;
+      const float4 a = *(const float4*)src, c = *(const float4*)(src + 4);
+      sv[0] += a.x; sv[1] += a.y; sv[2] += a.z; sv[3] += a.w;
+      sv[4] += c.x; sv[5] += c.y; sv[6] += c.z; sv[7] += c.w;
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int row = it * ROWS_PER_IT + row0;
+      const bool ok = row < p.BS && piece < dpieces;
+      const vec16 v = vec16{raw[it].x, raw[it].y, raw[it].z, raw[it].w};
+      float e[8];
+      Unpack<T>::run(v, e);
+      float t = 0.f;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const float x = ok ? e[q] * rn[it] : 0.f;
+        t = fmaf(x, sv[q] - x, t);
+      }
+      t = pieces_sum<PIECES>(t);
+      if (piece == 0 && row < p.BS) l_sum[row] = t;
+    }
   }
-  __syncthreads();
 
-  const int row_blocks = p.BS / 32;
-  for (int rb = wave; rb < row_blocks; rb += kPageThreads / 64) {
+  // ---- Gram tiles: wave a owns row block a and the column blocks (a + d) mod n
+  const int nrb = p.BS / 32;
+  if (wave < nrb) {
+    const int a = wave;
     bf16x8_t ahi[KSB], alo[KSB];
     {
-      const char* arow = hi_pl + (rb * 32 + col) * ROWH + half * 16;
+      const char* arow = hi_pl + (a * 32 + col) * ROWH + half * 16;
 #pragma unroll
       for (int s = 0; s < KSB; ++s) {
         ahi[s] = *(const bf16x8_t*)(arow + s * 32);
         alo[s] = *(const bf16x8_t*)(arow + PLANE + s * 32);
       }
     }
-    float rsum[16], cval[16];
-    int ccol[16];
+    int dcol[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { rsum[r] = 0.f; cval[r] = 0.f; ccol[r] = -1; }
+    for (int r = 0; r < 16; ++r) dcol[r] = -1;
+    const int nd = nrb / 2 + ((nrb & 1) || a < nrb / 2 ? 1 : 0);   // distances 0 .. nd-1
 #pragma unroll 1
-    for (int cb = 0; cb < row_blocks; ++cb) {
+    for (int d = 0; d < nd; ++d) {
+      const int cb = a + d < nrb ? a + d : a + d - nrb;
       f32x16_t acc;
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[r] = 0.f;
@@ -635,45 +703,71 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
         }
       }
       const int cslot = cb * 32 + col;
-      if (cb == rb) {   // the diagonal (a key against itself) only lives in this block
+      if (d == 0) {
+        // the diagonal block: a key against itself counts as 0, and both (i, j) and (j, i) are
+        // in the tile, so only the row side is recorded
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if ((r >> 2) * 8 + half * 4 + (r & 3) == col) acc[r] = 0.f;
-      }
+        for (int r = 0; r < 16; ++r) {
+          const bool diag = (r >> 2) * 8 + half * 4 + (r & 3) == col;
+          const float s = diag ? 0.f : acc[r];
+          dcol[r] = max(dcol[r], s > p.threshold ? cslot : -1);
+        }
+      } else {
+        // row side: key (a, r) sees column cslot; column side: key cslot sees the rows of block
+        // a, whose index grows with r inside a lane, so the last hit is the largest
+        int rlast = -1;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float s = acc[r];
-        rsum[r] += s;
-        if (s > p.threshold) { ccol[r] = cslot; cval[r] = s; }
+        for (int r = 0; r < 16; ++r) {
+          const bool over = acc[r] > p.threshold;
+          dcol[r] = max(dcol[r], over ? cslot : -1);
+          rlast = over ? r : rlast;
+        }
+        if (__any(rlast >= 0)) {
+          int ci = rlast < 0 ? -1 : a * 32 + (rlast >> 2) * 8 + half * 4 + (rlast & 3);
+          ci = max(ci, lane_xor32(ci));
+          if (half == 0 && ci >= 0) atomicMax(&l_col[cslot], ci);
+        }
       }
     }
-    // most waves see no entry over the threshold: then the (column, value) reduction is skipped
+    // most waves see no entry over the threshold: then the reduction over the lanes is skipped
     bool mine = false;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) mine |= ccol[r] >= 0;
-    const bool any_claim = __any(mine);
+    for (int r = 0; r < 16; ++r) mine |= dcol[r] >= 0;
+    if (__any(mine)) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      float s = rsum[r];
-      int c = ccol[r];
-      float v = cval[r];
-      s = half_sum(s);
-      if (any_claim) last_claim_reduce(c, v);
-      if (col == 0) {
-        const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-        l_sum[rslot] = s;
-        l_col[rslot] = c;
-        l_val[rslot] = v;
+      for (int r = 0; r < 16; ++r) {
+        const int c = half_max_i(dcol[r]);
+        if (col == 0 && c >= 0)
+          atomicMax(&l_col[a * 32 + (r >> 2) * 8 + half * 4 + (r & 3)], c);
       }
+    }
+  }
+  __syncthreads();
+  // ---- value of every key's claimed entry, from both planes: 16 lanes per key
+  __shared__ uint32_t claimed[kPageRows / 32];
+  if (tid < kPageRows / 32) claimed[tid] = 0u;
+  {
+    const int piece = tid % PIECES, g = tid / PIECES;
+#pragma unroll 1
+    for (int j = g; j < p.BS; j += kPageThreads / PIECES) {
+      const int c = l_col[j];
+      if (c < 0) continue;      // uniform over the 16 lanes of a key
+      const bf16x8_t hj = *(const bf16x8_t*)(hi_pl + j * ROWH + piece * 16);
+      const bf16x8_t lj = *(const bf16x8_t*)(lo_pl + j * ROWH + piece * 16);
+      const bf16x8_t hc = *(const bf16x8_t*)(hi_pl + c * ROWH + piece * 16);
+      const bf16x8_t lc = *(const bf16x8_t*)(lo_pl + c * ROWH + piece * 16);
+      float t = 0.f;
+#pragma unroll
+      for (int q = 0; q < 8; ++q)
+        t = fmaf((float)hj[q] + (float)lj[q], (float)hc[q] + (float)lc[q], t);
+      t = pieces_sum<PIECES>(t);
+      if (piece == 0) l_val[j] = t;
     }
   }
   __syncthreads();
   // r_i = rowsum_i - sum of the entries other rows claimed from row i.  Claims usually land on
   // a few rows, so a presence mask lets every other row skip the scan; two threads share a row
   // (fixed split and order: deterministic sums).
-  __shared__ uint32_t claimed[kPageRows / 32];
-  if (tid < kPageRows / 32) claimed[tid] = 0u;
-  __syncthreads();
   if (tid < p.BS) {
     const int c = l_col[tid];
     if (c >= 0) atomicOr(&claimed[c >> 5], 1u << (c & 31));
@@ -818,7 +912,8 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
   const size_t tail = (RAW ? 0 : (size_t)a.BS * 12) + sizeof(int) * 2 * a.NB;
   if constexpr (T::bytes == 2 && !RAW) {
     if (a.BS <= kPageRows && a.BS % 32 == 0) {
-      const size_t smem = 2 * (size_t)kPageRows * ROWH + (size_t)kPageRows * 12;
+      const size_t smem = 2 * (size_t)kPageRows * ROWH + (size_t)kPageRows * 12 +
+                          (size_t)kPageWaves * kDmax * 4;
       if (hipFuncSetAttribute((const void*)gram_page_kernel<T>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
         zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
