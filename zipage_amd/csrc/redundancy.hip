@@ -532,6 +532,22 @@ constexpr int kPageThreads = 512;
 constexpr int kPageWaves = kPageThreads / 64;
 constexpr int kPageRows = 256;
 
+// Two floats to packed bf16 (round to nearest even) in one v_cvt_pk_bf16_f32.
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pk_bf16(float a, float b) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{a, b}, bf16x2_t));
+}
+// hi = bf16(x), lo = bf16(x - hi) for eight values, packed pairwise.
+__device__ __forceinline__ void split8_pk(const float* x, u32x4& hi, u32x4& lo) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t h = pk_bf16(x[2 * i], x[2 * i + 1]);
+    hi[i] = h;
+    lo[i] = pk_bf16(x[2 * i] - __uint_as_float(h << 16), x[2 * i + 1] - __uint_as_float(h & 0xffff0000u));
+  }
+}
+
 // Largest value over the 32 lanes of a wave half.
 __device__ __forceinline__ int half_max_i(int v) {
   v = max(v, dpp_row_ror<8>(v));
@@ -584,7 +600,7 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
     constexpr int ITERS = kPageRows / ROWS_PER_IT;
     // all loads of the page are in flight before the first one is consumed
     u32x4 raw[ITERS];
-    float rn[ITERS];
+    float rn[ITERS], sq[ITERS];
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int row = it * ROWS_PER_IT + row0;
@@ -599,26 +615,27 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
     for (int it = 0; it < ITERS; ++it) {
       const int row = it * ROWS_PER_IT + row0;
       const bool ok = row < p.BS && piece < dpieces;
+      if (!ok) raw[it] = u32x4{0u, 0u, 0u, 0u};     // lanes past the page or the head dim hold zeros
       const vec16 v = vec16{raw[it].x, raw[it].y, raw[it].z, raw[it].w};
       float e[8];
       Unpack<T>::run(v, e);
       float ss = 0.f;
-      if (ok) {
 #pragma unroll
-        for (int q = 0; q < 8; ++q) ss += e[q] * e[q];
-      }
+      for (int q = 0; q < 8; ++q) ss = fmaf(e[q], e[q], ss);
       ss = pieces_sum<PIECES>(ss);
-      rn[it] = 1.f / fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
-      bf16x8_t hi, lo;
+      // the quotient is split into 16 mantissa bits below: the 1-ulp reciprocal is exact enough
+      rn[it] = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr));
+      sq[it] = ss * rn[it] * rn[it];
 #pragma unroll
       for (int q = 0; q < 8; ++q) {
-        e[q] = ok ? e[q] * rn[it] : 0.f;
+        e[q] *= rn[it];
         cs[q] += e[q];
       }
-      split8(e, hi, lo);
+      u32x4 hi, lo;
+      split8_pk(e, hi, lo);
       if (row < p.BS) {
-        *(bf16x8_t*)(hi_pl + row * ROWH + piece * 16) = hi;
-        *(bf16x8_t*)(lo_pl + row * ROWH + piece * 16) = lo;
+        *(u32x4*)(hi_pl + row * ROWH + piece * 16) = hi;
+        *(u32x4*)(lo_pl + row * ROWH + piece * 16) = lo;
       }
     }
     // the four key rows a wave handles per iteration sit 16 lanes apart
@@ -633,7 +650,8 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
       *(float4*)(dst + 4) = make_float4(cs[4], cs[5], cs[6], cs[7]);
     }
     __syncthreads();
-    // summed key (fixed order over the waves), then every key's dot product with the rest
+    // summed key (fixed order over the waves), then every key's dot product with the rest:
+    // e_i . (S - e_i) = rn_i (k_i . S) - |e_i|^2
     float sv[8];
 #pragma unroll
     for (int q = 0; q < 8; ++q) sv[q] = 0.f;
@@ -647,18 +665,14 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int row = it * ROWS_PER_IT + row0;
-      const bool ok = row < p.BS && piece < dpieces;
       const vec16 v = vec16{raw[it].x, raw[it].y, raw[it].z, raw[it].w};
       float e[8];
       Unpack<T>::run(v, e);
       float t = 0.f;
 #pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        const float x = ok ? e[q] * rn[it] : 0.f;
-        t = fmaf(x, sv[q] - x, t);
-      }
+      for (int q = 0; q < 8; ++q) t = fmaf(e[q], sv[q], t);
       t = pieces_sum<PIECES>(t);
-      if (piece == 0 && row < p.BS) l_sum[row] = t;
+      if (piece == 0 && row < p.BS) l_sum[row] = t * rn[it] - sq[it];
     }
   }
 
