@@ -304,6 +304,25 @@ def test_lightning_redundancy(dev, dtype, thr):
         _ulp_close(gr, wr, dtype, ulps=2, frac_exact=0.9)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("nb_choices", [(1, 2), (3, 4), (5, 6), (7,)])
+def test_raw_redundancy_page_counts(dev, dtype, nb_choices):
+    """Sequences of 1..7 pages in one padded table: every assignment of page pairs to
+    workgroups (odd and even page counts, wrapped pairs) against the oracle."""
+    from zipage_amd.kernel import raw_redudancy_score
+    s = _setup(59 + nb_choices[0], dtype, L=1, B=3, Hkv=2, Hq=2, BS=64, nb_choices=nb_choices,
+               budget=1, num_pages=30)
+    base = torch.randn((1, 1, 1, 2, 128), generator=torch.Generator().manual_seed(7))
+    k = (s["k"].float() * 0.7 + base).to(dtype)
+    for thr in (0.35, 0.6):
+        wl, wr = O.raw_redudancy_score(k, s["enc"], threshold=thr, temperature=0.4,
+                                       return_logits=True, rounding="fp32")
+        gl, gr = raw_redudancy_score(k.to(dev), s["enc"].to(dev), threshold=thr, temperature=0.4,
+                                     return_logits=True)
+        _ulp_close(gl, wl, dtype, ulps=1, abs_floor=1e-2)
+        _ulp_close(gr, wr, dtype, ulps=4)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_raw_redundancy(dev, dtype):
     from zipage_amd.kernel import raw_redudancy_score

@@ -807,6 +807,413 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
   }
 }
 
+// ------------------------------------------------------------------ raw, 16-bit caches
+// All-pairs variant over the whole sequence.  Three launches share the symmetric scheme of the
+// page kernel above, with pages in the role of its 32-key blocks:
+//   1. raw_rowsum_kernel: one workgroup per (layer, sequence, head) sums the normalised keys of
+//      the sequence and writes every key's row sum  e_i . (S - e_i); claims start at "none".
+//   2. gram_raw_kernel: one workgroup per valid page a; it multiplies page a with the pages
+//      (a + d) mod n, d = 0..n/2, so every unordered pair of pages is done once, and records for
+//      the keys on both sides the last (logical) column over the threshold with integer
+//      atomic maxima (order-independent, so the result is deterministic).
+//   3. raw_claim_value_kernel: the fp32 value of every key's claimed entry.
+// The softmax kernel then subtracts the claimed values from the rows they were taken from.
+
+template <typename T>
+__global__ __launch_bounds__(512) void raw_rowsum_kernel(GramArgs p) {
+  static_assert(T::bytes == 2, "16-bit caches only");
+  constexpr int kT = 512, PIECES = kDmax / 8, GROUPS = kT / PIECES, UNR = 4;
+  extern __shared__ __align__(16) char smem[];
+  float* l_part = (float*)smem;                       // [waves][kDmax]
+  int* vpage = (int*)(l_part + (kT / 64) * kDmax);
+  int* vidx = vpage + p.NB;
+  __shared__ int nvalid_s;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int piece = tid % PIECES, g = tid / PIECES;
+  const int h = blockIdx.x % p.Hkv;
+  const int b = (blockIdx.x / p.Hkv) % p.B;
+  const int l = blockIdx.x / (p.Hkv * p.B);
+  const int Tn = p.NB * p.BS;
+  const int64_t obase = (int64_t)blockIdx.x * Tn;
+  const float epsr = Elem<T>::rnd(p.eps);
+  if (tid == 0) {
+    int n = 0;
+    for (int j = 0; j < p.NB; ++j) {
+      const int c = p.table[(int64_t)b * p.NB + j];
+      const int pid = page_is_pad(c) ? -1 : page_id(c);
+      if (pid >= 0 && pid < p.num_pages) { vpage[n] = pid; vidx[n] = j; ++n; }
+    }
+    nvalid_s = n;
+  }
+  __syncthreads();
+  const int nrows = nvalid_s * p.BS;
+  const int dpieces = p.D / 8;
+  const bool pok = piece < dpieces;
+  const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
+  const char* kbase = p.k + (l * p.k_sl) * 2 + (int64_t)h * p.D * 2 + (pok ? piece : 0) * 16;
+  auto key_ptr = [&](int r) {
+    const int vp = r / p.BS, slot = r - vp * p.BS;
+    return kbase + (int64_t)vpage[vp] * p.k_sp * 2 + (int64_t)slot * k_row;
+  };
+
+  float cs[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) cs[q] = 0.f;
+  for (int r0 = g; r0 < nrows; r0 += GROUPS * UNR) {
+    u32x4 raw[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int r = r0 + u * GROUPS;
+      raw[u] = *(const u32x4*)key_ptr(r < nrows ? r : 0);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const bool ok = pok && r0 + u * GROUPS < nrows;
+      if (!ok) raw[u] = u32x4{0u, 0u, 0u, 0u};
+      float e[8];
+      Unpack<T>::run(vec16{raw[u].x, raw[u].y, raw[u].z, raw[u].w}, e);
+      float ss = 0.f;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) ss = fmaf(e[q], e[q], ss);
+      ss = pieces_sum<PIECES>(ss);
+      const float rn = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr));
+#pragma unroll
+      for (int q = 0; q < 8; ++q) cs[q] = fmaf(e[q], rn, cs[q]);
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < 8; ++q) {
+    cs[q] += lane_xor16(cs[q]);
+    cs[q] += lane_xor32(cs[q]);
+  }
+  if (lane < PIECES) {
+    float* dst = l_part + wave * kDmax + piece * 8;
+    *(float4*)dst = make_float4(cs[0], cs[1], cs[2], cs[3]);
+    *(float4*)(dst + 4) = make_float4(cs[4], cs[5], cs[6], cs[7]);
+  }
+  __syncthreads();
+  float sv[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q) sv[q] = 0.f;
+#pragma unroll
+  for (int w = 0; w < kT / 64; ++w) {
+    const float* src = l_part + w * kDmax + piece * 8;
+    const float4 a = *(const float4*)src, c = *(const float4*)(src + 4);
+    sv[0] += a.x; sv[1] += a.y; sv[2] += a.z; sv[3] += a.w;
+    sv[4] += c.x; sv[5] += c.y; sv[6] += c.z; sv[7] += c.w;
+  }
+  for (int r0 = g; r0 < nrows; r0 += GROUPS * UNR) {
+    u32x4 raw[UNR];
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int r = r0 + u * GROUPS;
+      raw[u] = *(const u32x4*)key_ptr(r < nrows ? r : 0);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int r = r0 + u * GROUPS;
+      if (!pok) raw[u] = u32x4{0u, 0u, 0u, 0u};
+      float e[8];
+      Unpack<T>::run(vec16{raw[u].x, raw[u].y, raw[u].z, raw[u].w}, e);
+      float ss = 0.f, t = 0.f;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        ss = fmaf(e[q], e[q], ss);
+        t = fmaf(e[q], sv[q], t);
+      }
+      ss = pieces_sum<PIECES>(ss);
+      t = pieces_sum<PIECES>(t);
+      const float rn = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr));
+      if (piece == 0 && r < nrows) {
+        const int vp = r / p.BS, slot = r - vp * p.BS;
+        const int64_t oi = obase + (int64_t)vidx[vp] * p.BS + slot;
+        p.ws_sum[oi] = t * rn - ss * rn * rn;
+        p.ws_col[oi] = -1;
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
+  static_assert(T::bytes == 2, "16-bit caches only");
+  constexpr int kThreads = 512, kWaves = 8;
+  constexpr int PIECES = kDmax / 8;
+  constexpr int ROWS_PER_IT = kThreads / PIECES;    // 32
+  constexpr int STAGE_IT = TN / ROWS_PER_IT;        // 2
+  constexpr int NSUB = TN / 32;
+  constexpr int KSB = kDmax / 16;
+  constexpr int PLANE = TN * ROWH;
+
+  extern __shared__ __align__(16) char smem[];
+  char* buf0 = smem;                                // [hi plane][lo plane]
+  char* buf1 = smem + 2 * PLANE;
+  int* l_cside = (int*)(smem + 4 * PLANE);          // [2][TN] column-side claims of a tile
+  int* vpage = l_cside + 2 * TN;
+  int* vidx = vpage + p.NB;
+  __shared__ int nvalid_s, mine_s;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const int jp = blockIdx.x % p.NB;
+  const int h = (blockIdx.x / p.NB) % p.Hkv;
+  const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
+  const int l = blockIdx.x / (p.NB * p.Hkv * p.B);
+  const int Tn = p.NB * p.BS;
+  const int64_t obase = (((int64_t)l * p.B + b) * p.Hkv + h) * Tn;
+  const float epsr = Elem<T>::rnd(p.eps);
+
+  const int code = p.table[(int64_t)b * p.NB + jp];
+  int rpid = page_is_pad(code) ? -1 : page_id(code);
+  if (rpid >= p.num_pages) rpid = -1;
+  if (rpid < 0) return;
+  if (tid == 0) {
+    int n = 0, me = 0;
+    for (int j = 0; j < p.NB; ++j) {
+      const int c = p.table[(int64_t)b * p.NB + j];
+      const int pid = page_is_pad(c) ? -1 : page_id(c);
+      if (pid >= 0 && pid < p.num_pages) {
+        if (j == jp) me = n;
+        vpage[n] = pid; vidx[n] = j; ++n;
+      }
+    }
+    nvalid_s = n;
+    mine_s = me;
+  }
+  for (int i = tid; i < 4 * PLANE / 4; i += kThreads) ((uint32_t*)smem)[i] = 0u;
+  if (tid < 2 * TN) l_cside[tid] = -1;
+  __syncthreads();
+  const int nv = nvalid_s, ia = mine_s;
+  const int nd = nv / 2 + (((nv & 1) || ia < nv / 2) ? 1 : 0);   // page distances 0 .. nd-1
+  const int tiles_per_page = p.BS / TN;
+  const int ntiles = nd * tiles_per_page;
+  const int dpieces = p.D / 8;
+  const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
+  const char* kbase = p.k + (l * p.k_sl) * 2 + (int64_t)h * p.D * 2;
+
+  const int st_piece = tid % PIECES, st_row0 = tid / PIECES;
+  const bool st_ok = st_piece < dpieces;
+  u32x4 pre[STAGE_IT];
+  auto tile_page = [&](int tile, int& d, int& toff) {
+    d = tile / tiles_per_page;
+    toff = (tile - d * tiles_per_page) * TN;
+    const int ic = ia + d;
+    return ic < nv ? ic : ic - nv;
+  };
+  auto issue_loads = [&](int tile) {
+    int d, toff;
+    const int ic = tile_page(tile, d, toff);
+    const char* src = kbase + (int64_t)vpage[ic] * p.k_sp * 2 + (int64_t)toff * k_row +
+                      (st_ok ? st_piece : 0) * 16;
+#pragma unroll
+    for (int i = 0; i < STAGE_IT; ++i)
+      pre[i] = *(const u32x4*)(src + (int64_t)(st_row0 + i * ROWS_PER_IT) * k_row);
+  };
+  auto commit_loads = [&](char* buf) {
+#pragma unroll
+    for (int i = 0; i < STAGE_IT; ++i) {
+      const int row = st_row0 + i * ROWS_PER_IT;
+      if (!st_ok) pre[i] = u32x4{0u, 0u, 0u, 0u};
+      float e[8];
+      Unpack<T>::run(vec16{pre[i].x, pre[i].y, pre[i].z, pre[i].w}, e);
+      float ss = 0.f;
+#pragma unroll
+      for (int q = 0; q < 8; ++q) ss = fmaf(e[q], e[q], ss);
+      ss = pieces_sum<PIECES>(ss);
+      const float rn = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr));
+#pragma unroll
+      for (int q = 0; q < 8; ++q) e[q] *= rn;
+      u32x4 hi, lo;
+      split8_pk(e, hi, lo);
+      if (st_ok) {
+        *(u32x4*)(buf + row * ROWH + st_piece * 16) = hi;
+        *(u32x4*)(buf + PLANE + row * ROWH + st_piece * 16) = lo;
+      }
+    }
+  };
+  // Hands the column-side claims of a finished tile to the keys of its page and clears the slot.
+  auto flush_cside = [&](int tile) {
+    if (tid < TN) {
+      int d, toff;
+      const int ic = tile_page(tile, d, toff);
+      int* slot = l_cside + (tile & 1) * TN + tid;
+      const int v = *slot;
+      if (v >= 0) {
+        atomicMax(p.ws_col + obase + (int64_t)vidx[ic] * p.BS + toff + tid, v);
+        *slot = -1;
+      }
+    }
+  };
+
+  const int row_blocks = p.BS / 32;
+  const int NR = (row_blocks + kWaves - 1) / kWaves;
+  for (int rr = 0; rr < NR; ++rr) {
+    const int rb = rr * kWaves + wave;
+    const bool active = rb < row_blocks;
+    // ---- A fragments: this lane's key row; lane (row, half) holds k = 16 s + 8 half + i
+    bf16x8_t ahi[KSB], alo[KSB];
+    {
+      const int slot = (active ? rb : 0) * 32 + col;
+      const char* src = kbase + (int64_t)rpid * p.k_sp * 2 + (int64_t)slot * k_row;
+      float x[KSB][8];
+      float ss = 0.f;
+#pragma unroll
+      for (int s = 0; s < KSB; ++s) {
+        const int pc = 2 * s + half;
+        vec16 v = vec16{0u, 0u, 0u, 0u};
+        if (pc < dpieces) v = *(const vec16*)(src + pc * 16);
+        Unpack<T>::run(v, x[s]);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) ss = fmaf(x[s][q], x[s][q], ss);
+      }
+      ss += lane_xor32(ss);  // the other half of the row
+      const float rn = active ? __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr)) : 0.f;
+#pragma unroll
+      for (int s = 0; s < KSB; ++s) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) x[s][q] *= rn;
+        u32x4 hi, lo;
+        split8_pk(x[s], hi, lo);
+        ahi[s] = __builtin_bit_cast(bf16x8_t, hi);
+        alo[s] = __builtin_bit_cast(bf16x8_t, lo);
+      }
+    }
+    int dcol[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dcol[r] = -1;
+
+    if (ntiles > 0) { issue_loads(0); commit_loads(buf0); }
+    __syncthreads();
+    for (int tile = 0; tile < ntiles; ++tile) {
+      char* cur = (tile & 1) ? buf1 : buf0;
+      char* nxt = (tile & 1) ? buf0 : buf1;
+      if (tile + 1 < ntiles) issue_loads(tile + 1);
+      if (tile > 0) flush_cside(tile - 1);   // its slot is next written two tiles from now
+      int d, toff;
+      const int ic = tile_page(tile, d, toff);
+      const int jc = vidx[ic];
+      if (active) {
+#pragma unroll 1
+        for (int st = 0; st < NSUB; ++st) {
+          f32x16_t acc;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+          const char* brow = cur + (st * 32 + col) * ROWH + half * 16;
+#pragma unroll
+          for (int s0 = 0; s0 < KSB; s0 += 4) {
+            bf16x8_t bh[4], bl[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+              bh[s] = *(const bf16x8_t*)(brow + (s0 + s) * 32);
+              bl[s] = *(const bf16x8_t*)(brow + PLANE + (s0 + s) * 32);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[s0 + s], bh[s], acc, 0, 0, 0);
+              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[s0 + s], bl[s], acc, 0, 0, 0);
+              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo[s0 + s], bh[s], acc, 0, 0, 0);
+            }
+          }
+          const int cslot = toff + st * 32 + col;
+          const int cidx = jc * p.BS + cslot;
+          if (d == 0) {
+            // the page against itself: both (i, j) and (j, i) are computed, the row side is enough
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+              const float s = rslot == cslot ? 0.f : acc[r];
+              dcol[r] = max(dcol[r], s > p.threshold ? cidx : -1);
+            }
+          } else {
+            // row side: key (rb, r) sees column cidx; column side: key cidx sees the rows of this
+            // block, whose index grows with r inside a lane
+            int rlast = -1;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const bool over = acc[r] > p.threshold;
+              dcol[r] = max(dcol[r], over ? cidx : -1);
+              rlast = over ? r : rlast;
+            }
+            if (__any(rlast >= 0)) {
+              int ci = rlast < 0 ? -1
+                                 : jp * p.BS + rb * 32 + (rlast >> 2) * 8 + half * 4 + (rlast & 3);
+              ci = max(ci, lane_xor32(ci));
+              if (half == 0 && ci >= 0) atomicMax(&l_cside[(tile & 1) * TN + st * 32 + col], ci);
+            }
+          }
+        }
+      }
+      if (tile + 1 < ntiles) commit_loads(nxt);
+      __syncthreads();
+    }
+    if (ntiles > 0) flush_cside(ntiles - 1);
+    bool any_mine = false;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) any_mine |= dcol[r] >= 0;
+    if (__any(any_mine)) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int c = half_max_i(dcol[r]);
+        if (active && col == 0 && c >= 0)
+          atomicMax(p.ws_col + obase + (int64_t)jp * p.BS + rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3), c);
+      }
+    }
+    __syncthreads();   // the claim slots are clear again before the next round writes them
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void raw_claim_value_kernel(GramArgs p) {
+  static_assert(T::bytes == 2, "16-bit caches only");
+  constexpr int PIECES = kDmax / 8, GROUPS = kThreads / PIECES;
+  const int tid = threadIdx.x;
+  const int piece = tid % PIECES, g = tid / PIECES;
+  const int jp = blockIdx.x % p.NB;
+  const int h = (blockIdx.x / p.NB) % p.Hkv;
+  const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
+  const int l = blockIdx.x / (p.NB * p.Hkv * p.B);
+  const int Tn = p.NB * p.BS;
+  const int64_t obase = (((int64_t)l * p.B + b) * p.Hkv + h) * Tn;
+  const float epsr = Elem<T>::rnd(p.eps);
+  const int code = p.table[(int64_t)b * p.NB + jp];
+  int rpid = page_is_pad(code) ? -1 : page_id(code);
+  if (rpid >= p.num_pages) rpid = -1;
+  if (rpid < 0) return;
+  const bool pok = piece < p.D / 8;
+  const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
+  const char* kbase = p.k + (l * p.k_sl) * 2 + (int64_t)h * p.D * 2 + (pok ? piece : 0) * 16;
+  for (int slot = g; slot < p.BS; slot += GROUPS) {
+    const int64_t oi = obase + (int64_t)jp * p.BS + slot;
+    const int c = p.ws_col[oi];
+    if (c < 0 || c >= Tn) continue;     // uniform over the 16 lanes of a key
+    const int cp = c / p.BS, cs = c - cp * p.BS;
+    const int ccode = p.table[(int64_t)b * p.NB + cp];
+    const int cpid = page_is_pad(ccode) ? -1 : page_id(ccode);
+    if (cpid < 0 || cpid >= p.num_pages) continue;
+    u32x4 ra = *(const u32x4*)(kbase + (int64_t)rpid * p.k_sp * 2 + (int64_t)slot * k_row);
+    u32x4 rc = *(const u32x4*)(kbase + (int64_t)cpid * p.k_sp * 2 + (int64_t)cs * k_row);
+    if (!pok) { ra = u32x4{0u, 0u, 0u, 0u}; rc = ra; }
+    float ea[8], ec[8];
+    Unpack<T>::run(vec16{ra.x, ra.y, ra.z, ra.w}, ea);
+    Unpack<T>::run(vec16{rc.x, rc.y, rc.z, rc.w}, ec);
+    float sa = 0.f, sc = 0.f, t = 0.f;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      sa = fmaf(ea[q], ea[q], sa);
+      sc = fmaf(ec[q], ec[q], sc);
+      t = fmaf(ea[q], ec[q], t);
+    }
+    sa = pieces_sum<PIECES>(sa);
+    sc = pieces_sum<PIECES>(sc);
+    t = pieces_sum<PIECES>(t);
+    const float rna = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(sa)), epsr));
+    const float rnc = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(sc)), epsr));
+    if (piece == 0) p.ws_val[oi] = t * rna * rnc;
+  }
+}
+
 // ------------------------------------------------------------------ softmax epilogue
 // One workgroup per (layer, sequence, head) row of T logits:
 //   raw only: r_i = rowsum_i - sum_{j: c*(j)=i} v_j, pad pages -inf
@@ -938,7 +1345,22 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
       return ZP_OK;
     }
   }
-  if constexpr (T::bytes == 2) {
+  if constexpr (T::bytes == 2 && RAW) {
+    const size_t smem0 = (size_t)(512 / 64) * kDmax * 4 + sizeof(int) * 2 * a.NB;
+    const size_t smem1 = 4 * (size_t)TN * ROWH + sizeof(int) * 2 * TN + sizeof(int) * 2 * a.NB;
+    if (hipFuncSetAttribute((const void*)gram_raw_kernel<T>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1) != hipSuccess) {
+      zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem1);
+      return ZP_EHIP;
+    }
+    hipLaunchKernelGGL((raw_rowsum_kernel<T>), dim3((unsigned)((int64_t)L * a.B * a.Hkv)), dim3(512),
+                       smem0, st, a);
+    hipLaunchKernelGGL((gram_raw_kernel<T>), grid, dim3(512), smem1, st, a);
+    hipLaunchKernelGGL((raw_claim_value_kernel<T>), grid, dim3(kThreads), 0, st, a);
+    ZP_LAUNCH_CHECK();
+    return ZP_OK;
+  }
+  if constexpr (T::bytes == 2 && !RAW) {
     const size_t smem = 4 * (size_t)TN * ROWH + tail;
     const bool wide = a.BS / 32 > kWaves;   // more row blocks than 4 waves: use 8 and halve the passes
     const void* fn = wide ? (const void*)gram_split_kernel<T, RAW, 8> : (const void*)gram_split_kernel<T, RAW, 4>;
