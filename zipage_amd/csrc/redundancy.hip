@@ -779,31 +779,33 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
     }
   }
   __syncthreads();
-  // r_i = rowsum_i - sum of the entries other rows claimed from row i.  Claims usually land on
-  // a few rows, so a presence mask lets every other row skip the scan; two threads share a row
-  // (fixed split and order: deterministic sums).
+  // r_i = rowsum_i - sum of the entries other keys claimed from row i.  Claims usually land on
+  // a few rows: a presence mask names them, and a wave sums the claims on each named row of its
+  // 32-row block with all of its lanes (four list entries per lane, then a fixed reduction tree:
+  // deterministic sums).
   if (tid < p.BS) {
     const int c = l_col[tid];
     if (c >= 0) atomicOr(&claimed[c >> 5], 1u << (c & 31));
   }
   __syncthreads();
   {
-    const int i = tid >> 1, part = tid & 1;
+    uint32_t m = claimed[wave];
     float corr = 0.f;
-    const bool need = i < p.BS && ((claimed[i >> 5] >> (i & 31)) & 1u);
-    if (need) {
-      const int j0 = part * (kPageRows / 2);
-      for (int j = j0; j < j0 + kPageRows / 2 && j < p.BS; j += 4) {
-        const int4 c4 = *(const int4*)(l_col + j);
-        const float4 v4 = *(const float4*)(l_val + j);
-        if (c4.x == i) corr += v4.x;
-        if (c4.y == i) corr += v4.y;
-        if (c4.z == i) corr += v4.z;
-        if (c4.w == i) corr += v4.w;
+    if (m) {
+      const int4 c4 = *(const int4*)(l_col + lane * 4);
+      const float4 v4 = *(const float4*)(l_val + lane * 4);
+      while (m) {
+        const int bit = __builtin_ctz(m);
+        m &= m - 1;
+        const int i = wave * 32 + bit;
+        float sum = (c4.x == i ? v4.x : 0.f) + (c4.y == i ? v4.y : 0.f) +
+                    (c4.z == i ? v4.z : 0.f) + (c4.w == i ? v4.w : 0.f);
+        sum = wave_sum(sum);
+        if (lane == bit) corr = sum;
       }
     }
-    const float other = __shfl_xor(corr, 1, 64);
-    if (part == 0 && i < p.BS) Elem<T>::st(p.r_out, obase + i, l_sum[i] - (corr + other));
+    const int i = wave * 32 + lane;
+    if (lane < 32 && i < p.BS) Elem<T>::st(p.r_out, obase + i, l_sum[i] - corr);
   }
 }
 
@@ -1261,13 +1263,31 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
       cval[t] = ok ? ws_val[base + t] : 0.f;
     }
     __syncthreads();
-    // Claims usually land on few rows: mark them, and only marked rows scan the claim list.
-    // The mark lives in x[], which the row's own value overwrites below.
+    // Claims usually land on few rows: mark them, and a wave sums the claims on each marked row
+    // of its 64-row chunks with all of its lanes (fixed order: deterministic).  The mark lives in
+    // x[] and is replaced by the sum, which the row's own value overwrites below.
     for (int t = threadIdx.x; t < Tn; t += kThreads) x[t] = 0.f;
     __syncthreads();
     for (int t = threadIdx.x; t < Tn; t += kThreads) {
       const int c = ccol[t];
       if (c >= 0 && c < Tn) x[c] = 1.f;   // benign race: every writer stores the same value
+    }
+    __syncthreads();
+    const int lane = lane_id();
+    for (int t0 = wave_id() * 64; t0 < Tn; t0 += kThreads) {
+      const int mine = t0 + lane;
+      uint64_t m = __ballot(mine < Tn && x[mine] != 0.f);
+      float corr = 0.f;
+      while (m) {
+        const int bit = __builtin_ctzll(m);
+        m &= m - 1;
+        const int t = t0 + bit;
+        float sum = 0.f;
+        for (int j = lane; j < Tn; j += 64) sum += ccol[j] == t ? cval[j] : 0.f;
+        sum = wave_sum(sum);
+        if (lane == bit) corr = sum;
+      }
+      if (mine < Tn) x[mine] = corr;
     }
     __syncthreads();
   }
@@ -1278,12 +1298,7 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
       const int c = trow[t / BS];
       const int pid = page_is_pad(c) ? -1 : page_id(c);
       if (pid >= 0 && pid < num_pages) {
-        float corr = 0.f;
-        if (x[t] != 0.f) {
-          for (int j = 0; j < Tn; ++j)
-            if (ccol[j] == t) corr += cval[j];
-        }
-        r = Elem<T>::rnd(ws_sum[base + t] - corr);
+        r = Elem<T>::rnd(ws_sum[base + t] - x[t]);
       } else {
         r = -INFINITY;
       }
