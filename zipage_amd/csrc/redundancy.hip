@@ -937,22 +937,22 @@ __global__ __launch_bounds__(512) void raw_rowsum_kernel(GramArgs p) {
   }
 }
 
-template <typename T>
+template <typename T, int TNc>
 __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
   static_assert(T::bytes == 2, "16-bit caches only");
   constexpr int kThreads = 512, kWaves = 8;
   constexpr int PIECES = kDmax / 8;
   constexpr int ROWS_PER_IT = kThreads / PIECES;    // 32
-  constexpr int STAGE_IT = TN / ROWS_PER_IT;        // 2
-  constexpr int NSUB = TN / 32;
+  constexpr int STAGE_IT = TNc / ROWS_PER_IT;        // 2
+  constexpr int NSUB = TNc / 32;
   constexpr int KSB = kDmax / 16;
-  constexpr int PLANE = TN * ROWH;
+  constexpr int PLANE = TNc * ROWH;
 
   extern __shared__ __align__(16) char smem[];
   char* buf0 = smem;                                // [hi plane][lo plane]
   char* buf1 = smem + 2 * PLANE;
-  int* l_cside = (int*)(smem + 4 * PLANE);          // [2][TN] column-side claims of a tile
-  int* vpage = l_cside + 2 * TN;
+  int* l_cside = (int*)(smem + 4 * PLANE);          // [2][TNc] column-side claims of a tile
+  int* vpage = l_cside + 2 * TNc;
   int* vidx = vpage + p.NB;
   __shared__ int nvalid_s, mine_s;
 
@@ -984,11 +984,11 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
     mine_s = me;
   }
   for (int i = tid; i < 4 * PLANE / 4; i += kThreads) ((uint32_t*)smem)[i] = 0u;
-  if (tid < 2 * TN) l_cside[tid] = -1;
+  if (tid < 2 * TNc) l_cside[tid] = -1;
   __syncthreads();
   const int nv = nvalid_s, ia = mine_s;
   const int nd = nv / 2 + (((nv & 1) || ia < nv / 2) ? 1 : 0);   // page distances 0 .. nd-1
-  const int tiles_per_page = p.BS / TN;
+  const int tiles_per_page = p.BS / TNc;
   const int ntiles = nd * tiles_per_page;
   const int dpieces = p.D / 8;
   const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
@@ -999,7 +999,7 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
   u32x4 pre[STAGE_IT];
   auto tile_page = [&](int tile, int& d, int& toff) {
     d = tile / tiles_per_page;
-    toff = (tile - d * tiles_per_page) * TN;
+    toff = (tile - d * tiles_per_page) * TNc;
     const int ic = ia + d;
     return ic < nv ? ic : ic - nv;
   };
@@ -1036,10 +1036,10 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
   };
   // Hands the column-side claims of a finished tile to the keys of its page and clears the slot.
   auto flush_cside = [&](int tile) {
-    if (tid < TN) {
+    if (tid < TNc) {
       int d, toff;
       const int ic = tile_page(tile, d, toff);
-      int* slot = l_cside + (tile & 1) * TN + tid;
+      int* slot = l_cside + (tile & 1) * TNc + tid;
       const int v = *slot;
       if (v >= 0) {
         atomicMax(p.ws_col + obase + (int64_t)vidx[ic] * p.BS + toff + tid, v);
@@ -1142,7 +1142,7 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
               int ci = rlast < 0 ? -1
                                  : jp * p.BS + rb * 32 + (rlast >> 2) * 8 + half * 4 + (rlast & 3);
               ci = max(ci, lane_xor32(ci));
-              if (half == 0 && ci >= 0) atomicMax(&l_cside[(tile & 1) * TN + st * 32 + col], ci);
+              if (half == 0 && ci >= 0) atomicMax(&l_cside[(tile & 1) * TNc + st * 32 + col], ci);
             }
           }
         }
@@ -1362,15 +1362,18 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
   }
   if constexpr (T::bytes == 2 && RAW) {
     const size_t smem0 = (size_t)(512 / 64) * kDmax * 4 + sizeof(int) * 2 * a.NB;
-    const size_t smem1 = 4 * (size_t)TN * ROWH + sizeof(int) * 2 * TN + sizeof(int) * 2 * a.NB;
-    if (hipFuncSetAttribute((const void*)gram_raw_kernel<T>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1) != hipSuccess) {
+    // column tiles of 128 keys when the page size allows: half as many workgroup barriers
+    const int tn = a.BS % 128 == 0 ? 128 : TN;
+    const size_t smem1 = 4 * (size_t)tn * ROWH + sizeof(int) * 2 * tn + sizeof(int) * 2 * a.NB;
+    const void* fn = tn == 128 ? (const void*)gram_raw_kernel<T, 128> : (const void*)gram_raw_kernel<T, TN>;
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1) != hipSuccess) {
       zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem1);
       return ZP_EHIP;
     }
     hipLaunchKernelGGL((raw_rowsum_kernel<T>), dim3((unsigned)((int64_t)L * a.B * a.Hkv)), dim3(512),
                        smem0, st, a);
-    hipLaunchKernelGGL((gram_raw_kernel<T>), grid, dim3(512), smem1, st, a);
+    if (tn == 128) hipLaunchKernelGGL((gram_raw_kernel<T, 128>), grid, dim3(512), smem1, st, a);
+    else hipLaunchKernelGGL((gram_raw_kernel<T, TN>), grid, dim3(512), smem1, st, a);
     hipLaunchKernelGGL((raw_claim_value_kernel<T>), grid, dim3(kThreads), 0, st, a);
     ZP_LAUNCH_CHECK();
     return ZP_OK;
