@@ -153,6 +153,11 @@ def main():
     ap.add_argument("--script-switches", action="store_true",
                     help="end-to-end leg: compress with the switch set of the reference's scripts "
                          "(global score, lightning redundancy, pooling) instead of pooling alone")
+    ap.add_argument("--pipeline-switches", choices=["pooling", "scripts", "raw"], default="pooling",
+                    help="compression switches of the single-layer leg: pooling alone (default, the "
+                         "headline line), the reference scripts' set (window 16, global score, "
+                         "lightning redundancy, pooling 5) or raw all-pairs redundancy with pooling 7; "
+                         "the non-default sets say so in config.workload")
     ap.add_argument("--ragged-prompts", action="store_true",
                     help="end-to-end leg: prompt lengths uniform in [P/2, 3P/2] so sequences reach "
                          "their budget on different steps")
@@ -193,10 +198,12 @@ def main():
             "config": {"workload": e2e["workload"]}, "roofline": e2e["decode_attention"],
             "cpu_baseline": None, "end_to_end": e2e}))
         return
+    sw = args.pipeline_switches
     if args.config == 2:
         batch, layers = args.batch or 64, 1
-        wl = ragged_batch(batch, L=1, pool_pages=20000, budget=8, W=32, seed=1,
-                          lengths=(2049, 2304), name="cfg2")
+        wl = ragged_batch(batch, L=1, pool_pages=20000, budget=8, W=16 if sw == "scripts" else 32,
+                          seed=1, lengths=(2049, 2304), name="cfg2",
+                          with_score_cache=sw == "scripts", compressed=sw == "scripts")
         desc = (f"configs[1]: {batch} ragged sequences, 1 layer, Qwen3-8B attention shape (32q/8kv "
                 "heads, head_dim 128), bf16, 9 pages x 256 tokens, window 32, 20k-page pool, score "
                 "-> max-pool 7 -> top-2048/head -> compact to 8 pages")
@@ -209,6 +216,19 @@ def main():
                 "pages (copy-on-write targets), 60k-page pool, Qwen3-8B shape, bf16, 36 layers run "
                 "one layer at a time over the same pool")
     cfg = CompressConfig(budget_blocks=8, query_cache_len=32, enable_pooling=True, pooling_size=7)
+    if sw != "pooling":
+        if args.config != 2:
+            sys.exit("bench.py: --pipeline-switches applies to --config 2")
+        if sw == "scripts":
+            cfg = CompressConfig(budget_blocks=8, query_cache_len=16, use_global_score=True,
+                                 decay_factor=0.8, use_redudancy=True, lightning_redudancy=True,
+                                 enable_pooling=True)
+            desc += (" [NOT the headline switches: window 16, global score (decay 0.8), lightning "
+                     "redundancy, max-pool 5, sequences already compressed once]")
+        else:
+            cfg = CompressConfig(budget_blocks=8, query_cache_len=32, use_redudancy=True,
+                                 lightning_redudancy=False, enable_pooling=True, pooling_size=7)
+            desc += " [NOT the headline switches: raw all-pairs redundancy added]"
 
     def step(timer=None):
         for _ in range(layers):
@@ -272,7 +292,7 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl, cfg, args.cpu_sample)
-    if not args.no_e2e and args.config == 2 and args.batch is None:
+    if not args.no_e2e and args.config == 2 and args.batch is None and sw == "pooling":
         del wl
         torch.cuda.empty_cache()
         out["end_to_end"] = end_to_end(args.requests, args.prompt, args.out_tokens,

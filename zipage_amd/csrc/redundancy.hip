@@ -548,6 +548,15 @@ __device__ __forceinline__ void split8_pk(const float* x, u32x4& hi, u32x4& lo) 
   }
 }
 
+// A similarity as 2^-32 fixed point (two's complement in an unsigned 64-bit word) and back: sums of
+// such words are exact and independent of the order of the additions.
+__device__ __forceinline__ unsigned long long to_fixed32(float v) {
+  return (unsigned long long)(long long)(v * 4294967296.f);
+}
+__device__ __forceinline__ float from_fixed32(unsigned long long w) {
+  return (float)(long long)w * (1.f / 4294967296.f);
+}
+
 // Largest value over the 32 lanes of a wave half.
 __device__ __forceinline__ int half_max_i(int v) {
   v = max(v, dpp_row_ror<8>(v));
@@ -567,9 +576,9 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
   extern __shared__ __align__(16) char smem[];
   char* hi_pl = smem;
   char* lo_pl = smem + PLANE;
-  float* l_sum = (float*)(smem + 2 * PLANE);
-  float* l_val = l_sum + kPageRows;
-  int* l_col = (int*)(l_val + kPageRows);
+  unsigned long long* l_corr = (unsigned long long*)(smem + 2 * PLANE);   // claimed from a row
+  float* l_sum = (float*)(l_corr + kPageRows);
+  int* l_col = (int*)(l_sum + kPageRows);
   float* l_part = (float*)(l_col + kPageRows);     // [waves][kDmax] partial key sums
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -607,7 +616,7 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
       raw[it] = *(const u32x4*)(page + (int64_t)(row < p.BS ? row : 0) * k_row +
                                 (piece < dpieces ? piece : 0) * 16);
     }
-    if (tid < kPageRows) l_col[tid] = -1;
+    if (tid < kPageRows) { l_col[tid] = -1; l_corr[tid] = 0ull; }
     float cs[8];
 #pragma unroll
     for (int q = 0; q < 8; ++q) cs[q] = 0.f;
@@ -757,9 +766,10 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
     }
   }
   __syncthreads();
-  // ---- value of every key's claimed entry, from both planes: 16 lanes per key
-  __shared__ uint32_t claimed[kPageRows / 32];
-  if (tid < kPageRows / 32) claimed[tid] = 0u;
+  // ---- value of every key's claimed entry, from both planes (16 lanes per key), subtracted from
+  // the row it was taken from.  Several keys may claim from one row: the values are added as
+  // 2^-32 fixed point with integer atomics, which is exact for a cosine above 2^-8 and does not
+  // depend on the order of the additions.
   {
     const int piece = tid % PIECES, g = tid / PIECES;
 #pragma unroll 1
@@ -775,38 +785,11 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
       for (int q = 0; q < 8; ++q)
         t = fmaf((float)hj[q] + (float)lj[q], (float)hc[q] + (float)lc[q], t);
       t = pieces_sum<PIECES>(t);
-      if (piece == 0) l_val[j] = t;
+      if (piece == 0) atomicAdd(&l_corr[c], to_fixed32(t));
     }
   }
   __syncthreads();
-  // r_i = rowsum_i - sum of the entries other keys claimed from row i.  Claims usually land on
-  // a few rows: a presence mask names them, and a wave sums the claims on each named row of its
-  // 32-row block with all of its lanes (four list entries per lane, then a fixed reduction tree:
-  // deterministic sums).
-  if (tid < p.BS) {
-    const int c = l_col[tid];
-    if (c >= 0) atomicOr(&claimed[c >> 5], 1u << (c & 31));
-  }
-  __syncthreads();
-  {
-    uint32_t m = claimed[wave];
-    float corr = 0.f;
-    if (m) {
-      const int4 c4 = *(const int4*)(l_col + lane * 4);
-      const float4 v4 = *(const float4*)(l_val + lane * 4);
-      while (m) {
-        const int bit = __builtin_ctz(m);
-        m &= m - 1;
-        const int i = wave * 32 + bit;
-        float sum = (c4.x == i ? v4.x : 0.f) + (c4.y == i ? v4.y : 0.f) +
-                    (c4.z == i ? v4.z : 0.f) + (c4.w == i ? v4.w : 0.f);
-        sum = wave_sum(sum);
-        if (lane == bit) corr = sum;
-      }
-    }
-    const int i = wave * 32 + lane;
-    if (lane < 32 && i < p.BS) Elem<T>::st(p.r_out, obase + i, l_sum[i] - corr);
-  }
+  if (tid < p.BS) Elem<T>::st(p.r_out, obase + tid, l_sum[tid] - from_fixed32(l_corr[tid]));
 }
 
 // ------------------------------------------------------------------ raw, 16-bit caches
@@ -1240,9 +1223,9 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
   extern __shared__ __align__(16) char smem[];
   __shared__ float red_lds[kWaves];
   const int Tn = NB * BS;
-  float* x = (float*)smem;          // [Tn]
-  int* ccol = (int*)(x + Tn);       // [Tn] raw only
-  float* cval = (float*)(ccol + (RAW ? Tn : 0));
+  // raw: [Tn] 64-bit sums of the values claimed from each row, then the [Tn] floats of the row
+  unsigned long long* corr = (unsigned long long*)smem;
+  float* x = (float*)(smem + (RAW ? (size_t)Tn * 8 : 0));
   const int64_t row = blockIdx.x;
   const int b = (int)((row / Hkv) % B);
   const int64_t base = row * Tn;
@@ -1255,39 +1238,16 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
   }
   const float divisor = RAW ? tscale * (float)(nvalid * BS) : tscale;
   if (RAW) {
+    // every key hands the value of its claimed entry to the row it was taken from: 2^-32 fixed
+    // point with integer atomics, exact and independent of the order
+    for (int t = threadIdx.x; t < Tn; t += kThreads) corr[t] = 0ull;
+    __syncthreads();
     for (int t = threadIdx.x; t < Tn; t += kThreads) {
       const int c = trow[t / BS];
       const int pid = page_is_pad(c) ? -1 : page_id(c);
-      const bool ok = pid >= 0 && pid < num_pages;
-      ccol[t] = ok ? ws_col[base + t] : -1;
-      cval[t] = ok ? ws_val[base + t] : 0.f;
-    }
-    __syncthreads();
-    // Claims usually land on few rows: mark them, and a wave sums the claims on each marked row
-    // of its 64-row chunks with all of its lanes (fixed order: deterministic).  The mark lives in
-    // x[] and is replaced by the sum, which the row's own value overwrites below.
-    for (int t = threadIdx.x; t < Tn; t += kThreads) x[t] = 0.f;
-    __syncthreads();
-    for (int t = threadIdx.x; t < Tn; t += kThreads) {
-      const int c = ccol[t];
-      if (c >= 0 && c < Tn) x[c] = 1.f;   // benign race: every writer stores the same value
-    }
-    __syncthreads();
-    const int lane = lane_id();
-    for (int t0 = wave_id() * 64; t0 < Tn; t0 += kThreads) {
-      const int mine = t0 + lane;
-      uint64_t m = __ballot(mine < Tn && x[mine] != 0.f);
-      float corr = 0.f;
-      while (m) {
-        const int bit = __builtin_ctzll(m);
-        m &= m - 1;
-        const int t = t0 + bit;
-        float sum = 0.f;
-        for (int j = lane; j < Tn; j += 64) sum += ccol[j] == t ? cval[j] : 0.f;
-        sum = wave_sum(sum);
-        if (lane == bit) corr = sum;
-      }
-      if (mine < Tn) x[mine] = corr;
+      if (pid < 0 || pid >= num_pages) continue;
+      const int cc = ws_col[base + t];
+      if (cc >= 0 && cc < Tn) atomicAdd(&corr[cc], to_fixed32(ws_val[base + t]));
     }
     __syncthreads();
   }
@@ -1298,7 +1258,7 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
       const int c = trow[t / BS];
       const int pid = page_is_pad(c) ? -1 : page_id(c);
       if (pid >= 0 && pid < num_pages) {
-        r = Elem<T>::rnd(ws_sum[base + t] - x[t]);
+        r = Elem<T>::rnd(ws_sum[base + t] - from_fixed32(corr[t]));
       } else {
         r = -INFINITY;
       }
@@ -1348,7 +1308,7 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
   const size_t tail = (RAW ? 0 : (size_t)a.BS * 12) + sizeof(int) * 2 * a.NB;
   if constexpr (T::bytes == 2 && !RAW) {
     if (a.BS <= kPageRows && a.BS % 32 == 0) {
-      const size_t smem = 2 * (size_t)kPageRows * ROWH + (size_t)kPageRows * 12 +
+      const size_t smem = 2 * (size_t)kPageRows * ROWH + (size_t)kPageRows * 16 +
                           (size_t)kPageWaves * kDmax * 4;
       if (hipFuncSetAttribute((const void*)gram_page_kernel<T>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
