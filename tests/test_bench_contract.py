@@ -17,5 +17,5 @@ def test_help_lists_the_contract_flags():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--help"],
                        capture_output=True, text=True, timeout=60)
     assert r.returncode == 0
-    for flag in ("--gpus", "--steps", "--warmup", "--config", "--no-e2e"):
+    for flag in ("--gpus", "--steps", "--warmup", "--config", "--no-e2e", "--pipeline-switches"):
         assert flag in r.stdout
