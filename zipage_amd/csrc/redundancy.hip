@@ -566,19 +566,40 @@ __device__ __forceinline__ int half_max_i(int v) {
   return max(v, lane_xor16(v));
 }
 
+// The 16-bit MFMA of the cache dtype: products of cache elements are exact in fp32.
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+template <typename T> struct Mfma16;
+template <> struct Mfma16<BF16> {
+  typedef bf16x8_t V;
+  __device__ static __forceinline__ f32x16_t run(V a, V b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct Mfma16<F16> {
+  typedef f16x8_t V;
+  __device__ static __forceinline__ f32x16_t run(V a, V b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+// The cosine matrix factors as S_ij = rn_i rn_j (k_i . k_j) with rn = 1 / norm: the raw 16-bit
+// keys go to the matrix cores as they are (one MFMA per k-step, exact products, fp32 sums) and
+// the two scale factors are applied to the accumulators.  One plane of raw keys in LDS (68 KB),
+// so two workgroups share a compute unit and one's page load hides behind the other's tiles.
 template <typename T>
 __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
   static_assert(T::bytes == 2, "16-bit caches only");
+  typedef typename Mfma16<T>::V frag_t;
   constexpr int PIECES = kDmax / 8;
   constexpr int KSB = kDmax / 16;
   constexpr int PLANE = kPageRows * ROWH;
 
   extern __shared__ __align__(16) char smem[];
-  char* hi_pl = smem;
-  char* lo_pl = smem + PLANE;
-  unsigned long long* l_corr = (unsigned long long*)(smem + 2 * PLANE);   // claimed from a row
+  char* k_pl = smem;                                                          // raw keys
+  unsigned long long* l_corr = (unsigned long long*)(smem + PLANE);           // claimed from a row
   float* l_sum = (float*)(l_corr + kPageRows);
-  int* l_col = (int*)(l_sum + kPageRows);
+  float* l_rn = l_sum + kPageRows;                                            // 1 / norm
+  int* l_col = (int*)(l_rn + kPageRows);
   float* l_part = (float*)(l_col + kPageRows);     // [waves][kDmax] partial key sums
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -602,7 +623,7 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
   const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
   const char* page = p.k + (l * p.k_sl + (int64_t)rpid * p.k_sp) * 2 + (int64_t)h * p.D * 2;
 
-  // ---- stage: normalise and split every key of the page, sum the normalised keys
+  // ---- stage: copy the page, norms, sum of the normalised keys, row sums
   {
     const int piece = tid % PIECES, row0 = tid / PIECES;       // 32 rows per iteration
     constexpr int ROWS_PER_IT = kPageThreads / PIECES;
@@ -625,27 +646,19 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
       const int row = it * ROWS_PER_IT + row0;
       const bool ok = row < p.BS && piece < dpieces;
       if (!ok) raw[it] = u32x4{0u, 0u, 0u, 0u};     // lanes past the page or the head dim hold zeros
-      const vec16 v = vec16{raw[it].x, raw[it].y, raw[it].z, raw[it].w};
+      if (row < p.BS) *(u32x4*)(k_pl + row * ROWH + piece * 16) = raw[it];
       float e[8];
-      Unpack<T>::run(v, e);
+      Unpack<T>::run(vec16{raw[it].x, raw[it].y, raw[it].z, raw[it].w}, e);
       float ss = 0.f;
 #pragma unroll
       for (int q = 0; q < 8; ++q) ss = fmaf(e[q], e[q], ss);
       ss = pieces_sum<PIECES>(ss);
-      // the quotient is split into 16 mantissa bits below: the 1-ulp reciprocal is exact enough
+      // the quotient only scales fp32 sums: the 1-ulp reciprocal is exact enough
       rn[it] = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr));
       sq[it] = ss * rn[it] * rn[it];
+      if (piece == 0 && row < p.BS) l_rn[row] = rn[it];
 #pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        e[q] *= rn[it];
-        cs[q] += e[q];
-      }
-      u32x4 hi, lo;
-      split8_pk(e, hi, lo);
-      if (row < p.BS) {
-        *(u32x4*)(hi_pl + row * ROWH + piece * 16) = hi;
-        *(u32x4*)(lo_pl + row * ROWH + piece * 16) = lo;
-      }
+      for (int q = 0; q < 8; ++q) cs[q] = fmaf(e[q], rn[it], cs[q]);
     }
     // the four key rows a wave handles per iteration sit 16 lanes apart
 #pragma unroll
@@ -674,9 +687,8 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int row = it * ROWS_PER_IT + row0;
-      const vec16 v = vec16{raw[it].x, raw[it].y, raw[it].z, raw[it].w};
       float e[8];
-      Unpack<T>::run(v, e);
+      Unpack<T>::run(vec16{raw[it].x, raw[it].y, raw[it].z, raw[it].w}, e);
       float t = 0.f;
 #pragma unroll
       for (int q = 0; q < 8; ++q) t = fmaf(e[q], sv[q], t);
@@ -689,15 +701,18 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
   const int nrb = p.BS / 32;
   if (wave < nrb) {
     const int a = wave;
-    bf16x8_t ahi[KSB], alo[KSB];
+    frag_t ak[KSB];
+    float rn_row[16];
     {
-      const char* arow = hi_pl + (a * 32 + col) * ROWH + half * 16;
+      const char* arow = k_pl + (a * 32 + col) * ROWH + half * 16;
 #pragma unroll
-      for (int s = 0; s < KSB; ++s) {
-        ahi[s] = *(const bf16x8_t*)(arow + s * 32);
-        alo[s] = *(const bf16x8_t*)(arow + PLANE + s * 32);
-      }
+      for (int s = 0; s < KSB; ++s) ak[s] = *(const frag_t*)(arow + s * 32);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) rn_row[r] = l_rn[a * 32 + (r >> 2) * 8 + half * 4 + (r & 3)];
     }
+    // a tile whose largest entry stays below this cannot hold a claim (slack for the rounding of
+    // the two ways the scale factors are multiplied in)
+    const float thr_lo = p.threshold - fabsf(p.threshold) * 1e-5f - 1e-30f;
     int dcol[16];
 #pragma unroll
     for (int r = 0; r < 16; ++r) dcol[r] = -1;
@@ -708,48 +723,41 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
       f32x16_t acc;
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-      const char* brow = hi_pl + (cb * 32 + col) * ROWH + half * 16;
-#pragma unroll
-      for (int s0 = 0; s0 < KSB; s0 += 4) {
-        bf16x8_t bh[4], bl[4];
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          bh[s] = *(const bf16x8_t*)(brow + (s0 + s) * 32);
-          bl[s] = *(const bf16x8_t*)(brow + PLANE + (s0 + s) * 32);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[s0 + s], bh[s], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[s0 + s], bl[s], acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo[s0 + s], bh[s], acc, 0, 0, 0);
-        }
-      }
+      const char* brow = k_pl + (cb * 32 + col) * ROWH + half * 16;
       const int cslot = cb * 32 + col;
+      const float rn_col = l_rn[cslot];
+      {
+        frag_t bk[KSB];
+#pragma unroll
+        for (int s = 0; s < KSB; ++s) bk[s] = *(const frag_t*)(brow + s * 32);
+#pragma unroll
+        for (int s = 0; s < KSB; ++s) acc = Mfma16<T>::run(ak[s], bk[s], acc);
+      }
       if (d == 0) {
-        // the diagonal block: a key against itself counts as 0, and both (i, j) and (j, i) are
-        // in the tile, so only the row side is recorded
+        // the diagonal block: a key against itself counts as 0
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const bool diag = (r >> 2) * 8 + half * 4 + (r & 3) == col;
-          const float s = diag ? 0.f : acc[r];
-          dcol[r] = max(dcol[r], s > p.threshold ? cslot : -1);
-        }
-      } else {
-        // row side: key (a, r) sees column cslot; column side: key cslot sees the rows of block
-        // a, whose index grows with r inside a lane, so the last hit is the largest
-        int rlast = -1;
+        for (int r = 0; r < 16; ++r)
+          if ((r >> 2) * 8 + half * 4 + (r & 3) == col) acc[r] = 0.f;
+      }
+      // most tiles hold no entry over the threshold: one maximum decides
+      float big = -INFINITY;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const bool over = acc[r] > p.threshold;
-          dcol[r] = max(dcol[r], over ? cslot : -1);
-          rlast = over ? r : rlast;
-        }
-        if (__any(rlast >= 0)) {
-          int ci = rlast < 0 ? -1 : a * 32 + (rlast >> 2) * 8 + half * 4 + (rlast & 3);
-          ci = max(ci, lane_xor32(ci));
-          if (half == 0 && ci >= 0) atomicMax(&l_col[cslot], ci);
-        }
+      for (int r = 0; r < 16; ++r) big = fmaxf(big, acc[r] * rn_row[r]);
+      if (!__any(big * rn_col > thr_lo)) continue;
+      // row side: key (a, r) sees column cslot; column side (off the diagonal block, where both
+      // (i, j) and (j, i) are computed): key cslot sees the rows of block a, whose index grows
+      // with r inside a lane, so the last hit is the largest
+      int rlast = -1;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const bool over = acc[r] * (rn_row[r] * rn_col) > p.threshold;
+        dcol[r] = max(dcol[r], over ? cslot : -1);
+        rlast = over ? r : rlast;
+      }
+      if (d != 0 && __any(rlast >= 0)) {
+        int ci = rlast < 0 ? -1 : a * 32 + (rlast >> 2) * 8 + half * 4 + (rlast & 3);
+        ci = max(ci, lane_xor32(ci));
+        if (half == 0 && ci >= 0) atomicMax(&l_col[cslot], ci);
       }
     }
     // most waves see no entry over the threshold: then the reduction over the lanes is skipped
@@ -766,26 +774,26 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
     }
   }
   __syncthreads();
-  // ---- value of every key's claimed entry, from both planes (16 lanes per key), subtracted from
-  // the row it was taken from.  Several keys may claim from one row: the values are added as
-  // 2^-32 fixed point with integer atomics, which is exact for a cosine above 2^-8 and does not
-  // depend on the order of the additions.
+  // ---- value of every key's claimed entry (16 lanes per key), subtracted from the row it was
+  // taken from.  Several keys may claim from one row: the values are added as 2^-32 fixed point
+  // with integer atomics, which is exact for a cosine above 2^-8 and does not depend on the order
+  // of the additions.
   {
     const int piece = tid % PIECES, g = tid / PIECES;
 #pragma unroll 1
     for (int j = g; j < p.BS; j += kPageThreads / PIECES) {
       const int c = l_col[j];
       if (c < 0) continue;      // uniform over the 16 lanes of a key
-      const bf16x8_t hj = *(const bf16x8_t*)(hi_pl + j * ROWH + piece * 16);
-      const bf16x8_t lj = *(const bf16x8_t*)(lo_pl + j * ROWH + piece * 16);
-      const bf16x8_t hc = *(const bf16x8_t*)(hi_pl + c * ROWH + piece * 16);
-      const bf16x8_t lc = *(const bf16x8_t*)(lo_pl + c * ROWH + piece * 16);
+      const u32x4 kj = *(const u32x4*)(k_pl + j * ROWH + piece * 16);
+      const u32x4 kc = *(const u32x4*)(k_pl + c * ROWH + piece * 16);
+      float ej[8], ec[8];
+      Unpack<T>::run(vec16{kj.x, kj.y, kj.z, kj.w}, ej);
+      Unpack<T>::run(vec16{kc.x, kc.y, kc.z, kc.w}, ec);
       float t = 0.f;
 #pragma unroll
-      for (int q = 0; q < 8; ++q)
-        t = fmaf((float)hj[q] + (float)lj[q], (float)hc[q] + (float)lc[q], t);
+      for (int q = 0; q < 8; ++q) t = fmaf(ej[q], ec[q], t);
       t = pieces_sum<PIECES>(t);
-      if (piece == 0) atomicAdd(&l_corr[c], to_fixed32(t));
+      if (piece == 0) atomicAdd(&l_corr[c], to_fixed32(t * (l_rn[j] * l_rn[c])));
     }
   }
   __syncthreads();
@@ -1308,7 +1316,7 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
   const size_t tail = (RAW ? 0 : (size_t)a.BS * 12) + sizeof(int) * 2 * a.NB;
   if constexpr (T::bytes == 2 && !RAW) {
     if (a.BS <= kPageRows && a.BS % 32 == 0) {
-      const size_t smem = 2 * (size_t)kPageRows * ROWH + (size_t)kPageRows * 16 +
+      const size_t smem = (size_t)kPageRows * ROWH + (size_t)kPageRows * 20 +
                           (size_t)kPageWaves * kDmax * 4;
       if (hipFuncSetAttribute((const void*)gram_page_kernel<T>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
