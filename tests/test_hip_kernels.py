@@ -304,6 +304,30 @@ def test_lightning_redundancy(dev, dtype, thr):
         _ulp_close(gr, wr, dtype, ulps=2, frac_exact=0.9)
 
 
+@pytest.mark.parametrize("dtype,scale", [(torch.float16, 2e-5), (torch.float16, 40.0),
+                                         (torch.bfloat16, 1e-12), (torch.bfloat16, 1e12)])
+@pytest.mark.parametrize("variant", ["lightning", "raw"])
+def test_redundancy_key_magnitudes(dev, dtype, scale, variant):
+    """The kernels multiply the keys as stored and scale afterwards: keys far from unit norm
+    (fp16 subnormal elements included) must give the same cosines as normalising first."""
+    from zipage_amd import kernel as K
+    s = _setup(71, dtype, L=1, B=2, Hkv=2, Hq=2, BS=64, nb_choices=(2, 3), budget=1, num_pages=12)
+    base = torch.randn((1, 1, 1, 2, 128), generator=torch.Generator().manual_seed(9))
+    k = ((s["k"].float() * 0.7 + base) * scale).to(dtype)
+    if variant == "lightning":
+        wl, wr = O.lightning_redudancy_score(k, s["enc"], threshold=0.45, temperature=0.4,
+                                             return_logits=True)
+        gl, gr = K.lightning_redudancy_score(k.to(dev), s["enc"].to(dev), threshold=0.45,
+                                             temperature=0.4, return_logits=True)
+    else:
+        wl, wr = O.raw_redudancy_score(k, s["enc"], threshold=0.45, temperature=0.4,
+                                       return_logits=True, rounding="fp32")
+        gl, gr = K.raw_redudancy_score(k.to(dev), s["enc"].to(dev), threshold=0.45,
+                                       temperature=0.4, return_logits=True)
+    _ulp_close(gl, wl, dtype, ulps=1, abs_floor=1e-2)
+    _ulp_close(gr, wr, dtype, ulps=4)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("nb_choices", [(1, 2), (3, 4), (5, 6), (7,)])
 def test_raw_redundancy_page_counts(dev, dtype, nb_choices):

@@ -923,6 +923,7 @@ __global__ __launch_bounds__(512) void raw_rowsum_kernel(GramArgs p) {
         const int64_t oi = obase + (int64_t)vidx[vp] * p.BS + slot;
         p.ws_sum[oi] = t * rn - ss * rn * rn;
         p.ws_col[oi] = -1;
+        p.ws_val[oi] = rn;      // read by the Gram kernel, replaced by the claim values after it
       }
     }
   }
@@ -931,18 +932,20 @@ __global__ __launch_bounds__(512) void raw_rowsum_kernel(GramArgs p) {
 template <typename T, int TNc>
 __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
   static_assert(T::bytes == 2, "16-bit caches only");
+  typedef typename Mfma16<T>::V frag_t;
   constexpr int kThreads = 512, kWaves = 8;
   constexpr int PIECES = kDmax / 8;
   constexpr int ROWS_PER_IT = kThreads / PIECES;    // 32
-  constexpr int STAGE_IT = TNc / ROWS_PER_IT;        // 2
+  constexpr int STAGE_IT = TNc / ROWS_PER_IT;
   constexpr int NSUB = TNc / 32;
   constexpr int KSB = kDmax / 16;
   constexpr int PLANE = TNc * ROWH;
 
   extern __shared__ __align__(16) char smem[];
-  char* buf0 = smem;                                // [hi plane][lo plane]
-  char* buf1 = smem + 2 * PLANE;
-  int* l_cside = (int*)(smem + 4 * PLANE);          // [2][TNc] column-side claims of a tile
+  char* buf0 = smem;                                // raw keys of a column tile
+  char* buf1 = smem + PLANE;
+  float* l_rn = (float*)(smem + 2 * PLANE);         // [2][TNc] 1 / norm of the tile's keys
+  int* l_cside = (int*)(l_rn + 2 * TNc);            // [2][TNc] column-side claims of a tile
   int* vpage = l_cside + 2 * TNc;
   int* vidx = vpage + p.NB;
   __shared__ int nvalid_s, mine_s;
@@ -955,7 +958,6 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
   const int l = blockIdx.x / (p.NB * p.Hkv * p.B);
   const int Tn = p.NB * p.BS;
   const int64_t obase = (((int64_t)l * p.B + b) * p.Hkv + h) * Tn;
-  const float epsr = Elem<T>::rnd(p.eps);
 
   const int code = p.table[(int64_t)b * p.NB + jp];
   int rpid = page_is_pad(code) ? -1 : page_id(code);
@@ -974,7 +976,8 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
     nvalid_s = n;
     mine_s = me;
   }
-  for (int i = tid; i < 4 * PLANE / 4; i += kThreads) ((uint32_t*)smem)[i] = 0u;
+  // head dims below 128 leave the upper pieces of every LDS row at zero
+  for (int i = tid; i < 2 * PLANE / 4; i += kThreads) ((uint32_t*)smem)[i] = 0u;
   if (tid < 2 * TNc) l_cside[tid] = -1;
   __syncthreads();
   const int nv = nvalid_s, ia = mine_s;
@@ -984,10 +987,12 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
   const int dpieces = p.D / 8;
   const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
   const char* kbase = p.k + (l * p.k_sl) * 2 + (int64_t)h * p.D * 2;
+  const float* rn_all = p.ws_val + obase;           // written by raw_rowsum_kernel
 
   const int st_piece = tid % PIECES, st_row0 = tid / PIECES;
   const bool st_ok = st_piece < dpieces;
   u32x4 pre[STAGE_IT];
+  float pre_rn = 0.f;
   auto tile_page = [&](int tile, int& d, int& toff) {
     d = tile / tiles_per_page;
     toff = (tile - d * tiles_per_page) * TNc;
@@ -1002,28 +1007,15 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
 #pragma unroll
     for (int i = 0; i < STAGE_IT; ++i)
       pre[i] = *(const u32x4*)(src + (int64_t)(st_row0 + i * ROWS_PER_IT) * k_row);
+    if (tid < TNc) pre_rn = rn_all[vidx[ic] * p.BS + toff + tid];
   };
-  auto commit_loads = [&](char* buf) {
+  auto commit_loads = [&](char* buf, int tile) {
+    if (st_ok) {
 #pragma unroll
-    for (int i = 0; i < STAGE_IT; ++i) {
-      const int row = st_row0 + i * ROWS_PER_IT;
-      if (!st_ok) pre[i] = u32x4{0u, 0u, 0u, 0u};
-      float e[8];
-      Unpack<T>::run(vec16{pre[i].x, pre[i].y, pre[i].z, pre[i].w}, e);
-      float ss = 0.f;
-#pragma unroll
-      for (int q = 0; q < 8; ++q) ss = fmaf(e[q], e[q], ss);
-      ss = pieces_sum<PIECES>(ss);
-      const float rn = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr));
-#pragma unroll
-      for (int q = 0; q < 8; ++q) e[q] *= rn;
-      u32x4 hi, lo;
-      split8_pk(e, hi, lo);
-      if (st_ok) {
-        *(u32x4*)(buf + row * ROWH + st_piece * 16) = hi;
-        *(u32x4*)(buf + PLANE + row * ROWH + st_piece * 16) = lo;
-      }
+      for (int i = 0; i < STAGE_IT; ++i)
+        *(u32x4*)(buf + (st_row0 + i * ROWS_PER_IT) * ROWH + st_piece * 16) = pre[i];
     }
+    if (tid < TNc) l_rn[(tile & 1) * TNc + tid] = pre_rn;
   };
   // Hands the column-side claims of a finished tile to the keys of its page and clears the slot.
   auto flush_cside = [&](int tile) {
@@ -1038,45 +1030,35 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
       }
     }
   };
+  const float thr_lo = p.threshold - fabsf(p.threshold) * 1e-5f - 1e-30f;
 
   const int row_blocks = p.BS / 32;
   const int NR = (row_blocks + kWaves - 1) / kWaves;
   for (int rr = 0; rr < NR; ++rr) {
     const int rb = rr * kWaves + wave;
     const bool active = rb < row_blocks;
-    // ---- A fragments: this lane's key row; lane (row, half) holds k = 16 s + 8 half + i
-    bf16x8_t ahi[KSB], alo[KSB];
+    // ---- A fragments: this lane's key row as stored; lane (row, half) holds k = 16 s + 8 half + i
+    frag_t ak[KSB];
+    float rn_row[16];
     {
       const int slot = (active ? rb : 0) * 32 + col;
       const char* src = kbase + (int64_t)rpid * p.k_sp * 2 + (int64_t)slot * k_row;
-      float x[KSB][8];
-      float ss = 0.f;
 #pragma unroll
       for (int s = 0; s < KSB; ++s) {
         const int pc = 2 * s + half;
-        vec16 v = vec16{0u, 0u, 0u, 0u};
-        if (pc < dpieces) v = *(const vec16*)(src + pc * 16);
-        Unpack<T>::run(v, x[s]);
-#pragma unroll
-        for (int q = 0; q < 8; ++q) ss = fmaf(x[s][q], x[s][q], ss);
+        u32x4 v = u32x4{0u, 0u, 0u, 0u};
+        if (pc < dpieces) v = *(const u32x4*)(src + pc * 16);
+        ak[s] = __builtin_bit_cast(frag_t, v);
       }
-      ss += lane_xor32(ss);  // the other half of the row
-      const float rn = active ? __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr)) : 0.f;
 #pragma unroll
-      for (int s = 0; s < KSB; ++s) {
-#pragma unroll
-        for (int q = 0; q < 8; ++q) x[s][q] *= rn;
-        u32x4 hi, lo;
-        split8_pk(x[s], hi, lo);
-        ahi[s] = __builtin_bit_cast(bf16x8_t, hi);
-        alo[s] = __builtin_bit_cast(bf16x8_t, lo);
-      }
+      for (int r = 0; r < 16; ++r)
+        rn_row[r] = rn_all[jp * p.BS + (active ? rb : 0) * 32 + (r >> 2) * 8 + half * 4 + (r & 3)];
     }
     int dcol[16];
 #pragma unroll
     for (int r = 0; r < 16; ++r) dcol[r] = -1;
 
-    if (ntiles > 0) { issue_loads(0); commit_loads(buf0); }
+    if (ntiles > 0) { issue_loads(0); commit_loads(buf0, 0); }
     __syncthreads();
     for (int tile = 0; tile < ntiles; ++tile) {
       char* cur = (tile & 1) ? buf1 : buf0;
@@ -1093,52 +1075,46 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[r] = 0.f;
           const char* brow = cur + (st * 32 + col) * ROWH + half * 16;
+          const float rn_col = l_rn[(tile & 1) * TNc + st * 32 + col];
+          {
+            frag_t bk[KSB];
 #pragma unroll
-          for (int s0 = 0; s0 < KSB; s0 += 4) {
-            bf16x8_t bh[4], bl[4];
+            for (int s = 0; s < KSB; ++s) bk[s] = *(const frag_t*)(brow + s * 32);
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-              bh[s] = *(const bf16x8_t*)(brow + (s0 + s) * 32);
-              bl[s] = *(const bf16x8_t*)(brow + PLANE + (s0 + s) * 32);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int s = 0; s < 4; ++s) {
-              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[s0 + s], bh[s], acc, 0, 0, 0);
-              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ahi[s0 + s], bl[s], acc, 0, 0, 0);
-              acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(alo[s0 + s], bh[s], acc, 0, 0, 0);
-            }
+            for (int s = 0; s < KSB; ++s) acc = Mfma16<T>::run(ak[s], bk[s], acc);
           }
           const int cslot = toff + st * 32 + col;
           const int cidx = jc * p.BS + cslot;
           if (d == 0) {
-            // the page against itself: both (i, j) and (j, i) are computed, the row side is enough
+            // the page against itself: a key against itself counts as 0
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-              const float s = rslot == cslot ? 0.f : acc[r];
-              dcol[r] = max(dcol[r], s > p.threshold ? cidx : -1);
-            }
-          } else {
-            // row side: key (rb, r) sees column cidx; column side: key cidx sees the rows of this
-            // block, whose index grows with r inside a lane
-            int rlast = -1;
+            for (int r = 0; r < 16; ++r)
+              if (rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3) == cslot) acc[r] = 0.f;
+          }
+          // most tiles hold no entry over the threshold: one maximum decides
+          float big = -INFINITY;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const bool over = acc[r] > p.threshold;
-              dcol[r] = max(dcol[r], over ? cidx : -1);
-              rlast = over ? r : rlast;
-            }
-            if (__any(rlast >= 0)) {
-              int ci = rlast < 0 ? -1
-                                 : jp * p.BS + rb * 32 + (rlast >> 2) * 8 + half * 4 + (rlast & 3);
-              ci = max(ci, lane_xor32(ci));
-              if (half == 0 && ci >= 0) atomicMax(&l_cside[(tile & 1) * TNc + st * 32 + col], ci);
-            }
+          for (int r = 0; r < 16; ++r) big = fmaxf(big, acc[r] * rn_row[r]);
+          if (!__any(big * rn_col > thr_lo)) continue;
+          // row side: key (rb, r) sees column cidx; column side (other pages only: inside a
+          // page both (i, j) and (j, i) are computed): key cidx sees the rows of this block,
+          // whose index grows with r inside a lane
+          int rlast = -1;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const bool over = acc[r] * (rn_row[r] * rn_col) > p.threshold;
+            dcol[r] = max(dcol[r], over ? cidx : -1);
+            rlast = over ? r : rlast;
+          }
+          if (d != 0 && __any(rlast >= 0)) {
+            int ci = rlast < 0 ? -1
+                               : jp * p.BS + rb * 32 + (rlast >> 2) * 8 + half * 4 + (rlast & 3);
+            ci = max(ci, lane_xor32(ci));
+            if (half == 0 && ci >= 0) atomicMax(&l_cside[(tile & 1) * TNc + st * 32 + col], ci);
           }
         }
       }
-      if (tile + 1 < ntiles) commit_loads(nxt);
+      if (tile + 1 < ntiles) commit_loads(nxt, tile + 1);
       __syncthreads();
     }
     if (ntiles > 0) flush_cside(ntiles - 1);
@@ -1332,7 +1308,7 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
     const size_t smem0 = (size_t)(512 / 64) * kDmax * 4 + sizeof(int) * 2 * a.NB;
     // column tiles of 128 keys when the page size allows: half as many workgroup barriers
     const int tn = a.BS % 128 == 0 ? 128 : TN;
-    const size_t smem1 = 4 * (size_t)tn * ROWH + sizeof(int) * 2 * tn + sizeof(int) * 2 * a.NB;
+    const size_t smem1 = 2 * (size_t)tn * ROWH + sizeof(int) * 4 * tn + sizeof(int) * 2 * a.NB;
     const void* fn = tn == 128 ? (const void*)gram_raw_kernel<T, 128> : (const void*)gram_raw_kernel<T, TN>;
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1) != hipSuccess) {
       zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem1);
