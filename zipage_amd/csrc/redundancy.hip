@@ -929,8 +929,12 @@ __global__ __launch_bounds__(512) void raw_rowsum_kernel(GramArgs p) {
   }
 }
 
+// Four waves per SIMD, i.e. two workgroups per compute unit (their LDS fits twice): one's barrier
+// and LDS waits hide behind the other's tiles.  The register cap spills a few addresses outside
+// the tile loop; measured 10-15 % faster than one workgroup per unit.
 template <typename T, int TNc>
-__global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(4, 4)))
+void gram_raw_kernel(GramArgs p) {
   static_assert(T::bytes == 2, "16-bit caches only");
   typedef typename Mfma16<T>::V frag_t;
   constexpr int kThreads = 512, kWaves = 8;
@@ -946,7 +950,8 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
   char* buf1 = smem + PLANE;
   float* l_rn = (float*)(smem + 2 * PLANE);         // [2][TNc] 1 / norm of the tile's keys
   int* l_cside = (int*)(l_rn + 2 * TNc);            // [2][TNc] column-side claims of a tile
-  int* vpage = l_cside + 2 * TNc;
+  float* l_rnrow = (float*)(l_cside + 2 * TNc);     // [BS] 1 / norm of the row page's keys
+  int* vpage = (int*)(l_rnrow + p.BS);
   int* vidx = vpage + p.NB;
   __shared__ int nvalid_s, mine_s;
 
@@ -979,6 +984,7 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
   // head dims below 128 leave the upper pieces of every LDS row at zero
   for (int i = tid; i < 2 * PLANE / 4; i += kThreads) ((uint32_t*)smem)[i] = 0u;
   if (tid < 2 * TNc) l_cside[tid] = -1;
+  for (int i = tid; i < p.BS; i += kThreads) l_rnrow[i] = p.ws_val[obase + (int64_t)jp * p.BS + i];
   __syncthreads();
   const int nv = nvalid_s, ia = mine_s;
   const int nd = nv / 2 + (((nv & 1) || ia < nv / 2) ? 1 : 0);   // page distances 0 .. nd-1
@@ -1039,7 +1045,7 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
     const bool active = rb < row_blocks;
     // ---- A fragments: this lane's key row as stored; lane (row, half) holds k = 16 s + 8 half + i
     frag_t ak[KSB];
-    float rn_row[16];
+    const float* rsrc = l_rnrow + (active ? rb : 0) * 32 + half * 4;   // this lane's 16 rows: 1 / norm
     {
       const int slot = (active ? rb : 0) * 32 + col;
       const char* src = kbase + (int64_t)rpid * p.k_sp * 2 + (int64_t)slot * k_row;
@@ -1050,9 +1056,6 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
         if (pc < dpieces) v = *(const u32x4*)(src + pc * 16);
         ak[s] = __builtin_bit_cast(frag_t, v);
       }
-#pragma unroll
-      for (int r = 0; r < 16; ++r)
-        rn_row[r] = rn_all[jp * p.BS + (active ? rb : 0) * 32 + (r >> 2) * 8 + half * 4 + (r & 3)];
     }
     int dcol[16];
 #pragma unroll
@@ -1076,12 +1079,19 @@ __global__ __launch_bounds__(512) void gram_raw_kernel(GramArgs p) {
           for (int r = 0; r < 16; ++r) acc[r] = 0.f;
           const char* brow = cur + (st * 32 + col) * ROWH + half * 16;
           const float rn_col = l_rn[(tile & 1) * TNc + st * 32 + col];
-          {
-            frag_t bk[KSB];
 #pragma unroll
-            for (int s = 0; s < KSB; ++s) bk[s] = *(const frag_t*)(brow + s * 32);
+          for (int s0 = 0; s0 < KSB; s0 += 4) {
+            frag_t bk[4];
 #pragma unroll
-            for (int s = 0; s < KSB; ++s) acc = Mfma16<T>::run(ak[s], bk[s], acc);
+            for (int s = 0; s < 4; ++s) bk[s] = *(const frag_t*)(brow + (s0 + s) * 32);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) acc = Mfma16<T>::run(ak[s0 + s], bk[s], acc);
+          }
+          float rn_row[16];
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const float4 v = *(const float4*)(rsrc + g * 8);
+            rn_row[4 * g] = v.x; rn_row[4 * g + 1] = v.y; rn_row[4 * g + 2] = v.z; rn_row[4 * g + 3] = v.w;
           }
           const int cslot = toff + st * 32 + col;
           const int cidx = jc * p.BS + cslot;
@@ -1308,7 +1318,8 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
     const size_t smem0 = (size_t)(512 / 64) * kDmax * 4 + sizeof(int) * 2 * a.NB;
     // column tiles of 128 keys when the page size allows: half as many workgroup barriers
     const int tn = a.BS % 128 == 0 ? 128 : TN;
-    const size_t smem1 = 2 * (size_t)tn * ROWH + sizeof(int) * 4 * tn + sizeof(int) * 2 * a.NB;
+    const size_t smem1 = 2 * (size_t)tn * ROWH + sizeof(int) * 4 * tn + sizeof(float) * a.BS +
+                         sizeof(int) * 2 * a.NB;
     const void* fn = tn == 128 ? (const void*)gram_raw_kernel<T, 128> : (const void*)gram_raw_kernel<T, TN>;
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1) != hipSuccess) {
       zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem1);
