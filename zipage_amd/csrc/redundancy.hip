@@ -4,15 +4,21 @@
 // threshold is zeroed too; the row sums are the redundancy logits.
 //
 // The Gram matrix is symmetric, so "last row over the threshold in column j" equals "last
-// column over the threshold in row j".  A wave owns 32 rows for all columns, tracks per
-// row the plain row sum and the last column over the threshold (with its value); the
-// claimed entries are subtracted afterwards from the rows they belong to:
+// column over the threshold in row j" (the key's claim); the claimed entries are subtracted
+// afterwards from the rows they were taken from:
 //     r_i = sum_j S_ij  -  sum_{j : c*(j) = i} S_ji .
-// This needs one pass over the columns and no cross-wave ordering.
 //
-// Arithmetic follows the reference: keys are divided by their cache-dtype norm in fp32 and
-// the dot products are fp32 (v_mfma_f32_32x32x2_f32, A = 32 key rows in registers,
-// B = 64-key column tiles normalised on the way into double-buffered LDS).
+// Kernels in this file:
+//   gram_kernel        fp32 caches, both variants: v_mfma_f32_32x32x2_f32 on keys divided by
+//                      their cache-dtype norm in fp32 (the reference's arithmetic), full
+//                      matrix, a wave owns 32 rows for all columns.
+//   gram_split_kernel  16-bit caches, lightning with pages above 256 keys: normalised keys
+//                      split into two bf16 planes, three MFMAs per k-step, full matrix.
+//   gram_page_kernel   16-bit caches, lightning: stored keys on the matrix cores, 1/norm
+//                      factors on the accumulators, every pair of key blocks once.
+//   raw_rowsum_kernel, gram_raw_kernel, raw_claim_value_kernel
+//                      16-bit caches, raw: the same over the pages of a sequence.
+//   red_softmax_kernel claim corrections of the raw variant and the softmax of both.
 #include "common.h"
 #include <math.h>
 
