@@ -328,6 +328,32 @@ def test_redundancy_key_magnitudes(dev, dtype, scale, variant):
     _ulp_close(gr, wr, dtype, ulps=4)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("BS,D", [(128, 128), (512, 128), (256, 64), (64, 32), (192, 128)])
+@pytest.mark.parametrize("variant", ["lightning", "raw"])
+def test_redundancy_page_and_head_sizes(dev, dtype, BS, D, variant):
+    """Page sizes on both sides of the 256-key page kernel (and one that is no multiple of 128)
+    and head dims below 128, which leave part of every staged key row at zero."""
+    from zipage_amd import kernel as K
+    s = _setup(83, dtype, L=1, B=2, Hkv=2, Hq=2, D=D, BS=BS, nb_choices=(2, 3), budget=1,
+               num_pages=10)
+    base = torch.randn((1, 1, 1, 2, D), generator=torch.Generator().manual_seed(11))
+    k = (s["k"].float() * 0.7 + base).to(dtype)
+    kw = dict(threshold=0.45, temperature=0.4, return_logits=True)
+    if variant == "lightning":
+        wl, wr = O.lightning_redudancy_score(k, s["enc"], **kw)
+        gl, gr = K.lightning_redudancy_score(k.to(dev), s["enc"].to(dev), **kw)
+    else:
+        wl, wr = O.raw_redudancy_score(k, s["enc"], rounding="reference" if dtype == torch.float32 else "fp32", **kw)
+        gl, gr = K.raw_redudancy_score(k.to(dev), s["enc"].to(dev), **kw)
+    if dtype == torch.float32:
+        _rel_close(gl, wl, rel=1e-4, abs_floor=1e-2)
+        _rel_close(gr, wr, rel=1e-3, abs_floor=1e-9)
+    else:
+        _ulp_close(gl, wl, dtype, ulps=1, abs_floor=1e-2)
+        _ulp_close(gr, wr, dtype, ulps=4)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("nb_choices", [(1, 2), (3, 4), (5, 6), (7,)])
 def test_raw_redundancy_page_counts(dev, dtype, nb_choices):
