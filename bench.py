@@ -164,6 +164,11 @@ def main():
     ap.add_argument("--separate-select-stages", action="store_true",
                     help="run pooling, the mask epilogue and top-k as three launches (timed under "
                          "the reference's stage names) instead of the one-launch selection")
+    ap.add_argument("--place-tries", type=int, default=4,
+                    help="K/V pool allocations to try before any data is written, keeping the one "
+                         "on which a small timed gather runs fastest (an engine allocates its pools "
+                         "once and can do the same); every probe figure is reported in "
+                         "'placement'; 1 = take the first allocation")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", type=int, default=64)
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -203,7 +208,8 @@ def main():
         batch, layers = args.batch or 64, 1
         wl = ragged_batch(batch, L=1, pool_pages=20000, budget=8, W=16 if sw == "scripts" else 32,
                           seed=1, lengths=(2049, 2304), name="cfg2",
-                          with_score_cache=sw == "scripts", compressed=sw == "scripts")
+                          with_score_cache=sw == "scripts", compressed=sw == "scripts",
+                          place_tries=args.place_tries)
         desc = (f"configs[1]: {batch} ragged sequences, 1 layer, Qwen3-8B attention shape (32q/8kv "
                 "heads, head_dim 128), bf16, 9 pages x 256 tokens, window 32, 20k-page pool, score "
                 "-> max-pool 7 -> top-2048/head -> compact to 8 pages")
@@ -211,7 +217,7 @@ def main():
         batch, layers = args.batch or 256, 36
         wl = ragged_batch(batch, L=1, pool_pages=60000, budget=8, W=32, seed=3,
                           lengths=(2049, 2560), shared_prefix_group=16, shared_prefix_pages=2,
-                          name="cfg4")
+                          name="cfg4", place_tries=args.place_tries)
         desc = (f"configs[3]: {batch} ragged sequences (9-10 pages), groups of 16 share 2 prefix "
                 "pages (copy-on-write targets), 60k-page pool, Qwen3-8B shape, bf16, 36 layers run "
                 "one layer at a time over the same pool")
@@ -290,6 +296,8 @@ def main():
                      "hbm_frac_of_stage_time": round(alg["pipeline"] / (gpu_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      "stages_ms": stages_ms},
     }
+    if wl.placement is not None:
+        out["placement"] = wl.placement
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl, cfg, args.cpu_sample)
     if not args.no_e2e and args.config == 2 and args.batch is None and sw == "pooling":

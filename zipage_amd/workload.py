@@ -30,6 +30,7 @@ class Workload:
     budget: int
     W: int
     tables: list
+    placement: dict | None = None  # report of placement.place_pools, when it chose the pools
 
     @property
     def B(self):
@@ -49,11 +50,13 @@ def encode_tables(tables, device):
 def ragged_batch(B, *, L=1, pool_pages=20000, budget=8, W=32, BS=256, dtype=torch.bfloat16,
                  seed=1, lengths=(2049, 2304), shared_prefix_group=0, shared_prefix_pages=2,
                  with_score_cache=False, compressed=False, shape=QWEN3_8B, device="cuda:0",
-                 name="ragged"):
+                 name="ragged", place_tries=1):
     """B sequences with token counts uniform in ``lengths`` (rounded up to whole pages, since
     compression fires only on a full last page), pages drawn without replacement from a pool
     of ``pool_pages`` ids.  With ``shared_prefix_group = n`` every group of n sequences shares
-    its first ``shared_prefix_pages`` pages (copy-on-write targets)."""
+    its first ``shared_prefix_pages`` pages (copy-on-write targets).  With ``place_tries > 1``
+    the K/V pools are placed by ``placement.place_pools`` (a timed gather on up to that many
+    fresh allocations, before any data is written); the report is kept in ``placement``."""
     g = torch.Generator().manual_seed(seed)
     Hq, Hkv, D = shape["Hq"], shape["Hkv"], shape["D"]
     lens = torch.randint(lengths[0], lengths[1] + 1, (B,), generator=g)
@@ -86,8 +89,22 @@ def ragged_batch(B, *, L=1, pool_pages=20000, budget=8, W=32, BS=256, dtype=torc
         targets.append(target)
     used = sorted({p for t in tables for p in t})
     dev = torch.device(device)
-    k = torch.empty((L, pool_pages, BS, Hkv, D), dtype=dtype, device=dev)
-    v = torch.empty((L, pool_pages, BS, Hkv, D), dtype=dtype, device=dev)
+    block_tables = encode_tables(tables, dev)
+    compressed_t = torch.full((B,), bool(compressed), dtype=torch.bool, device=dev)
+    targets_t = torch.tensor(targets, dtype=torch.int32, device=dev)
+
+    def alloc():
+        return (torch.empty((L, pool_pages, BS, Hkv, D), dtype=dtype, device=dev),
+                torch.empty((L, pool_pages, BS, Hkv, D), dtype=dtype, device=dev))
+
+    placement = None
+    if place_tries > 1:
+        from zipage_amd.placement import place_pools, probe_gather_us
+        (k, v), placement = place_pools(
+            alloc, lambda kv: probe_gather_us(kv[0], kv[1], block_tables, compressed_t, targets_t,
+                                              budget * BS), place_tries)
+    else:
+        k, v = alloc()
     gg = torch.Generator(device=dev).manual_seed(seed)
     idx = torch.tensor(used, device=dev)
     for l in range(L):
@@ -104,10 +121,8 @@ def ragged_batch(B, *, L=1, pool_pages=20000, budget=8, W=32, BS=256, dtype=torc
     return Workload(
         name=name, k=k, v=v, q=q, score_cache=sc,
         query_ids=torch.arange(B, dtype=torch.int32, device=dev),
-        block_tables=encode_tables(tables, dev),
-        compressed=torch.full((B,), bool(compressed), dtype=torch.bool, device=dev),
-        targets=torch.tensor(targets, dtype=torch.int32, device=dev),
-        budget=budget, W=W, tables=tables)
+        block_tables=block_tables, compressed=compressed_t, targets=targets_t,
+        budget=budget, W=W, tables=tables, placement=placement)
 
 
 def algorithmic_bytes(wl: Workload, cfg) -> dict:
