@@ -164,8 +164,8 @@ def main():
     ap.add_argument("--separate-select-stages", action="store_true",
                     help="run pooling, the mask epilogue and top-k as three launches (timed under "
                          "the reference's stage names) instead of the one-launch selection")
-    ap.add_argument("--place-tries", type=int, default=4,
-                    help="K/V pool allocations to try before any data is written, keeping the one "
+    ap.add_argument("--place-tries", type=int, default=6,
+                    help="K/V pool allocations to make side by side before any data is written, keeping the one "
                          "on which a small timed gather runs fastest (an engine allocates its pools "
                          "once and can do the same); every probe figure is reported in "
                          "'placement'; 1 = take the first allocation")
