@@ -164,11 +164,14 @@ def main():
     ap.add_argument("--separate-select-stages", action="store_true",
                     help="run pooling, the mask epilogue and top-k as three launches (timed under "
                          "the reference's stage names) instead of the one-launch selection")
-    ap.add_argument("--place-tries", type=int, default=6,
-                    help="K/V pool allocations to make side by side before any data is written, keeping the one "
-                         "on which a small timed gather runs fastest (an engine allocates its pools "
-                         "once and can do the same); every probe figure is reported in "
-                         "'placement'; 1 = take the first allocation")
+    ap.add_argument("--place-tries", type=int, default=16,
+                    help="most pool-sized allocations made side by side before any data is written "
+                         "(allocation stops as soon as a pair is fast or 160 GB are held); a small "
+                         "timed gather on pairs of them picks the K pool and the V pool (the "
+                         "in-place compaction is ~15 %% faster when the two lie in different regions "
+                         "of device memory; an engine allocates its pools once and can do the "
+                         "same); every probe figure is reported in 'placement'; 1 = take the first "
+                         "two allocations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", type=int, default=64)
     ap.add_argument("--calibrate-copy", action="store_true",

@@ -1,15 +1,16 @@
 """Choosing where the KV pools land in device memory.
 
-The in-place compaction (and every other gather through the page table) runs 10-15 % faster or
-slower depending on which physical region the driver gave the pool allocation; inside one
-allocation the figure never changes, and neither the page set a batch touches nor the distance
-between the K and V pools matters.  An engine allocates its pools once, so it can afford to
-time a small gather on a fresh allocation and try another region when the first one is slow.
-``place_pools`` does that; the candidates stay allocated until the choice is made, because a
-candidate allocated after another was released would land in the released region again (on a
-fresh device, 20 GB allocations made one after the other and all kept alive gave 202, 202, 203,
-180, 170, 196, 194, 197, 173 and 199 microseconds for the same gather, the same in every
-process).
+Measured on MI355X: device memory behaves as a few large physical zones (about 70, 100 and
+100+ GB in allocation order on a fresh device).  A kernel that reads and writes K and V at
+once -- the in-place compaction -- runs ~15 % faster when the K pool and the V pool lie in
+DIFFERENT zones (169 us against 194-197 us for 64 sequences), whatever the virtual addresses,
+alignment or physical chunking; striping either pool over zones gives the same 169 us.  A
+read-only kernel (decode attention) prefers K and V in the SAME zone by ~4 %.  Inside one
+allocation the figure never changes, and neither the page set a batch touches nor a small
+shift between the pools matters.  The driver gives no way to ask for a zone, but an engine
+allocates its pools once, so it can allocate a few pool-sized slabs side by side, time a small
+gather on pairs of them, keep the best pair and release the rest: ``place_kv_pools``.
+``place_pools`` is the simpler form for candidates that hold both pools.
 """
 from __future__ import annotations
 
@@ -59,3 +60,35 @@ def place_pools(alloc, probe, tries=6, good_enough=None):
     if torch.cuda.is_available():
         torch.cuda.empty_cache()
     return best, {"tries": len(times), "probe_us": times, "kept": kept}
+
+
+def place_kv_pools(alloc_one, probe_pair, slabs=16, gain=0.93, span_bytes=160e9, pool_bytes=None):
+    """``alloc_one() -> pool`` allocates ONE pool-sized tensor; ``probe_pair(k, v) ->
+    microseconds``.  Allocates pools side by side (all stay alive, so they cover consecutive
+    regions of device memory) and probes the first one as the K pool against each new one as
+    the V pool, until a pair runs in ``gain`` x the slowest pair's time or less (the new pool
+    reached another zone), ``slabs`` pools exist, their total passes ``span_bytes`` (needs
+    ``pool_bytes``) or memory runs out.  Returns ``((k, v), report)`` for the fastest pair; the
+    other pools are released."""
+    pools, times = [alloc_one()], {}
+    while len(pools) < max(2, slabs):
+        if pool_bytes is not None and len(pools) >= 2 and (len(pools) + 1) * pool_bytes > span_bytes:
+            break
+        try:
+            pools.append(alloc_one())
+        except torch.cuda.OutOfMemoryError:
+            break
+        j = len(pools) - 1
+        times[(0, j)] = round(probe_pair(pools[0], pools[j]), 1)
+        if min(times.values()) <= gain * max(times.values()):
+            break
+    if len(pools) < 2:
+        raise RuntimeError("place_kv_pools: fewer than two pools fit in device memory")
+    (ki, vi) = min(times, key=times.get)
+    k, v = pools[ki], pools[vi]
+    n = len(pools)
+    del pools
+    if torch.cuda.is_available():
+        torch.cuda.empty_cache()
+    return (k, v), {"slabs": n, "probe_us": {f"{i}-{j}": t for (i, j), t in times.items()},
+                    "kept": [ki, vi]}

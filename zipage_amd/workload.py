@@ -55,8 +55,9 @@ def ragged_batch(B, *, L=1, pool_pages=20000, budget=8, W=32, BS=256, dtype=torc
     compression fires only on a full last page), pages drawn without replacement from a pool
     of ``pool_pages`` ids.  With ``shared_prefix_group = n`` every group of n sequences shares
     its first ``shared_prefix_pages`` pages (copy-on-write targets).  With ``place_tries > 1``
-    the K/V pools are placed by ``placement.place_pools`` (a timed gather on up to that many
-    fresh allocations, before any data is written); the report is kept in ``placement``."""
+    the K and V pools are chosen by ``placement.place_kv_pools`` among that many pool-sized
+    allocations made side by side (a timed gather on pairs of them, before any data is
+    written); the report is kept in ``placement``."""
     g = torch.Generator().manual_seed(seed)
     Hq, Hkv, D = shape["Hq"], shape["Hkv"], shape["D"]
     lens = torch.randint(lengths[0], lengths[1] + 1, (B,), generator=g)
@@ -93,18 +94,18 @@ def ragged_batch(B, *, L=1, pool_pages=20000, budget=8, W=32, BS=256, dtype=torc
     compressed_t = torch.full((B,), bool(compressed), dtype=torch.bool, device=dev)
     targets_t = torch.tensor(targets, dtype=torch.int32, device=dev)
 
-    def alloc():
-        return (torch.empty((L, pool_pages, BS, Hkv, D), dtype=dtype, device=dev),
-                torch.empty((L, pool_pages, BS, Hkv, D), dtype=dtype, device=dev))
+    def alloc_one():
+        return torch.empty((L, pool_pages, BS, Hkv, D), dtype=dtype, device=dev)
 
     placement = None
     if place_tries > 1:
-        from zipage_amd.placement import place_pools, probe_gather_us
-        (k, v), placement = place_pools(
-            alloc, lambda kv: probe_gather_us(kv[0], kv[1], block_tables, compressed_t, targets_t,
-                                              budget * BS), place_tries)
+        from zipage_amd.placement import place_kv_pools, probe_gather_us
+        (k, v), placement = place_kv_pools(
+            alloc_one, lambda kp, vp: probe_gather_us(kp, vp, block_tables, compressed_t, targets_t,
+                                                      budget * BS), place_tries,
+            pool_bytes=L * pool_pages * BS * Hkv * D * torch.empty((), dtype=dtype).element_size())
     else:
-        k, v = alloc()
+        k, v = alloc_one(), alloc_one()
     gg = torch.Generator(device=dev).manual_seed(seed)
     idx = torch.tensor(used, device=dev)
     for l in range(L):
