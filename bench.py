@@ -16,6 +16,7 @@ decode engine and adds decode tokens/s and the compression share as `end_to_end`
 from __future__ import annotations
 
 import argparse
+import dataclasses
 import json
 import os
 import sys
@@ -47,9 +48,8 @@ def cpu_baseline(wl, cfg, sample_seqs, budget_s=30.0):
     for it in range(4):
         kk, vv = k.clone(), v.clone()
         t0 = time.perf_counter()
-        O.compress_pipeline(kk, vv, q, None, qid, enc, comp, tgt, budget_blocks=cfg.budget_blocks,
-                            query_cache_len=cfg.query_cache_len, enable_pooling=cfg.enable_pooling,
-                            pooling_size=cfg.pooling_size)
+        sc = None if sub["score_cache"] is None else sub["score_cache"].clone()
+        O.compress_pipeline(kk, vv, q, sc, qid, enc, comp, tgt, **dataclasses.asdict(cfg))
         dt = time.perf_counter() - t0
         if it > 0:
             times.append(dt)
@@ -137,9 +137,11 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--batch", type=int, default=None)
-    ap.add_argument("--config", type=int, default=2, choices=[2, 4, 5],
+    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5],
                     help="workload, numbered from 1 as in BASELINE.json: 2 = 64 ragged sequences, one "
-                         "layer (default, the headline line); 4 = 256 sequences with shared "
+                         "layer (default, the headline line); 3 = 128 sequences at Qwen3-0.6B "
+                         "shape in fp32 with the global-score and redundancy terms (lightning; "
+                         "--pipeline-switches raw for all pairs); 4 = 256 sequences with shared "
                          "prefixes and copy-on-write targets, 36 layers run one layer at a time "
                          "over one page pool; 5 = the end-to-end decode case alone")
     ap.add_argument("--no-e2e", action="store_true",
@@ -216,6 +218,17 @@ def main():
         desc = (f"configs[1]: {batch} ragged sequences, 1 layer, Qwen3-8B attention shape (32q/8kv "
                 "heads, head_dim 128), bf16, 9 pages x 256 tokens, window 32, 20k-page pool, score "
                 "-> max-pool 7 -> top-2048/head -> compact to 8 pages")
+    elif args.config == 3:
+        from zipage_amd.workload import QWEN3_0_6B
+        batch, layers = args.batch or 128, 1
+        wl = ragged_batch(batch, L=1, pool_pages=2048, budget=8, W=32, seed=0, lengths=(2304, 2304),
+                          dtype=torch.float32, shape=QWEN3_0_6B, name="cfg3", with_score_cache=True,
+                          compressed=True, place_tries=args.place_tries)
+        desc = (f"configs[2]: {batch} sequences, 1 layer, Qwen3-0.6B attention shape (16q/8kv heads, "
+                "head_dim 128), fp32, 9 pages x 256 tokens, window 32, 2048-page pool, score -> global "
+                "score (U(0,1) carried, decay 0.9, added) -> avg-pool 7 -> minus 0.5 x "
+                + ("raw all-pairs" if sw == "raw" else "lightning (same-page)")
+                + " redundancy (lambda 2/3) -> top-2048/head -> compact to 8 pages")
     else:
         batch, layers = args.batch or 256, 36
         wl = ragged_batch(batch, L=1, pool_pages=60000, budget=8, W=32, seed=3,
@@ -225,9 +238,17 @@ def main():
                 "pages (copy-on-write targets), 60k-page pool, Qwen3-8B shape, bf16, 36 layers run "
                 "one layer at a time over the same pool")
     cfg = CompressConfig(budget_blocks=8, query_cache_len=32, enable_pooling=True, pooling_size=7)
-    if sw != "pooling":
+    if args.config == 3:
+        if sw == "scripts":
+            sys.exit("bench.py: --config 3 takes --pipeline-switches pooling (lightning) or raw")
+        cfg = CompressConfig(budget_blocks=8, query_cache_len=32, use_global_score=True,
+                             decay_factor=0.9, activate_method="sum", use_redudancy=True,
+                             lightning_redudancy=sw != "raw", redudancy_lambda=2.0 / 3.0,
+                             enable_pooling=True, continues_pooling=True, pooling_size=7,
+                             pooling_mode="avg")
+    elif sw != "pooling":
         if args.config != 2:
-            sys.exit("bench.py: --pipeline-switches applies to --config 2")
+            sys.exit("bench.py: --pipeline-switches applies to --config 2 and 3")
         if sw == "scripts":
             cfg = CompressConfig(budget_blocks=8, query_cache_len=16, use_global_score=True,
                                  decay_factor=0.8, use_redudancy=True, lightning_redudancy=True,
@@ -285,13 +306,14 @@ def main():
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic",
+        "dtype": "f32" if args.config == 3 else "bf16", "data": "synthetic",
         "config": {"workload": desc, "batch": wl.B, "layers": layers},
         "roofline": {"bound": "hbm", "kernel": "compact_kernel (compress_kv)",
                      "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": args.traffic if args.traffic is not None
-                     else COMPACT_TRAFFIC_PER_SEQ_LAYER * wl.B,
+                     else (COMPACT_TRAFFIC_PER_SEQ_LAYER * wl.B if wl.k.element_size() == 2
+                           else None),   # the counter runs were made on the bf16 workloads
                      "algorithmic_bytes": alg["compress_kv"],
                      "avg_launch_us": round(kv_s * 1e6, 2)},
         "pipeline": {"algorithmic_bytes": alg["pipeline"],
@@ -302,7 +324,8 @@ def main():
     if wl.placement is not None:
         out["placement"] = wl.placement
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(wl, cfg, args.cpu_sample)
+        out["cpu_baseline"] = cpu_baseline(wl, cfg, min(args.cpu_sample, 16) if args.config == 3
+                                           else args.cpu_sample)
     if not args.no_e2e and args.config == 2 and args.batch is None and sw == "pooling":
         del wl
         torch.cuda.empty_cache()
