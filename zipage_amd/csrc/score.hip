@@ -7,7 +7,8 @@
 // three passes over the sequence's pages, recomputing QK^T each time:
 //   pass 1  row maximum of the (rounded) logits,
 //   pass 2  row sum of exp(rounded(logit - max)),
-//   pass 3  p = exp(.) / sum, max over the group, sum over the window, store.
+//   pass 3  p = exp(.) / sum, max over the group, sum over the window, store (the group
+//           maximum is taken on the exponents x*log2(e) - log2(sum), one exponential per group).
 // Passes 2 and 3 re-read K from L2 / Infinity Cache.  Rounding points follow the
 // reference (logits, logit-max, softmax output and the window mean are each rounded to the
 // cache dtype), so bf16/fp16 results agree with it to the last bit except where fp32
@@ -144,6 +145,14 @@ __device__ __forceinline__ float exp_neg(float x) {
   return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
 }
 
+// 2^y through the hardware exponential (y <= 0 here; -inf gives 0).
+__device__ __forceinline__ float exp2_hw(float y) {
+#ifdef ZP_DBG_NOEXP
+  return y;
+#endif
+  return __builtin_amdgcn_exp2f(y);
+}
+
 // GPC: padded GQA group size known at compile time (0: read it from the arguments); RMAXC: window
 // reduction known at compile time (0 mean, 1 max, -1: from the arguments).  The common shape
 // (group 4, mean) gets its own instantiation: straight-line epilogues instead of uniform branches
@@ -274,9 +283,9 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
     for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(afrag[s]));
     // rows owned by this lane in the accumulator layout: (r/4)*8 + half*4 + r%4
     const int row0 = rb * 32 + half * 4;
-    float invl[16], mx[16];
+    float cl[16], mx[16];   // cl = -log2(row sum): p = 2^(x*log2(e) + cl)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { mx[r] = 0.f; invl[r] = 0.f; }
+    for (int r = 0; r < 16; ++r) { mx[r] = 0.f; cl[r] = -INFINITY; }
 
     // One sweep over the sequence's K tiles.  PASS 0: row max; 1: row sum of exp; 2: output.
     auto sweep = [&](auto pass_c) {
@@ -379,15 +388,15 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
                 Rnd<T>::pair(s0, s1);
                 float x0 = s0 - mx[r], x1 = s1 - mx[r + 1];
                 Rnd<T>::pair(x0, x1);
-                const float e0 = exp_neg(x0), e1 = exp_neg(x1);
                 if constexpr (PASS == 1) {
-                  run[r] += e0;
-                  run[r + 1] += e1;
+                  run[r] += exp_neg(x0);
+                  run[r + 1] += exp_neg(x1);
                 } else {
-                  // rounding to the cache dtype is monotone, so max over the group of the rounded
-                  // probabilities == rounded max: groups of >= 2 rows round after their maximum
-                  pv[r] = e0 * invl[r];
-                  pv[r + 1] = e1 * invl[r + 1];
+                  // p = exp(x) / sum = 2^(x*log2(e) - log2(sum)).  The exponential and the rounding
+                  // to the cache dtype are monotone, so the maximum over the group is taken on the
+                  // exponents and a group of n rows costs one exponential and one rounding
+                  pv[r] = __builtin_fmaf(x0, 1.44269504088896340736f, cl[r]);
+                  pv[r + 1] = __builtin_fmaf(x1, 1.44269504088896340736f, cl[r + 1]);
                 }
               }
               if constexpr (PASS == 2) {
@@ -396,7 +405,11 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
                 const int Gp = GpV;
                 if (Gp < 2) {  // no group: every probability is rounded on its own
 #pragma unroll
-                  for (int r = 0; r < 16; r += 2) Rnd<T>::pair(pv[r], pv[r + 1]);
+                  for (int r = 0; r < 16; r += 2) {
+                    pv[r] = exp2_hw(pv[r]);
+                    pv[r + 1] = exp2_hw(pv[r + 1]);
+                    Rnd<T>::pair(pv[r], pv[r + 1]);
+                  }
                 }
                 if (Gp >= 4) {
                   float q4[4];
@@ -408,6 +421,8 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
                     for (int q = 0; q < 4; ++q) q4[q] = vmax(q4[q], lane_xor32(q4[q]));
                   }
                   if (Gp < 16) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) q4[q] = exp2_hw(q4[q]);
                     Rnd<T>::pair(q4[0], q4[1]);
                     Rnd<T>::pair(q4[2], q4[3]);
                   }
@@ -415,10 +430,12 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
                     q4[0] = vmax(q4[0], q4[1]);
                     q4[2] = vmax(q4[2], q4[3]);
                     if (Gp >= 32) {
-                      red = vmax(q4[0], q4[2]);
+                      red = exp2_hw(vmax(q4[0], q4[2]));
                       float dummy = red;
                       Rnd<T>::pair(red, dummy);
                     } else {
+                      q4[0] = exp2_hw(q4[0]);
+                      q4[2] = exp2_hw(q4[2]);
                       Rnd<T>::pair(q4[0], q4[2]);
                       red = rmaxV ? vmax(q4[0], q4[2]) : q4[0] + q4[2];
                     }
@@ -430,7 +447,7 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
                   float t8[8];
                   if (Gp == 2) {
 #pragma unroll
-                    for (int q = 0; q < 8; ++q) t8[q] = vmax(pv[2 * q], pv[2 * q + 1]);
+                    for (int q = 0; q < 8; ++q) t8[q] = exp2_hw(vmax(pv[2 * q], pv[2 * q + 1]));
 #pragma unroll
                     for (int q = 0; q < 8; q += 2) Rnd<T>::pair(t8[q], t8[q + 1]);
                   } else {
@@ -488,7 +505,7 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
           } else {
             const int m = row0 + (r >> 2) * 8 + (r & 3);
             const bool ok = active && (m >> gsV) < p.W && (m & (GpV - 1)) < p.G;
-            invl[r] = ok ? 1.f / v : 0.f;
+            cl[r] = ok ? -__builtin_amdgcn_logf(v) : -INFINITY;   // rows outside the window or group never win a maximum
           }
         }
         __syncthreads();
