@@ -182,11 +182,13 @@ __global__ __launch_bounds__(kThreads) void gram_kernel(GramArgs p) {
 #pragma unroll
       for (int q = 0; q < NE; ++q) ss += e[q] * e[q];
       ss = pieces_sum<PIECES>(ss);
-      const float n = fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
+      // one reciprocal per key and a multiplication per element (the hardware square root and
+      // reciprocal are each within 1 ulp; a division per element would dominate the staging)
+      const float rn = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(__builtin_amdgcn_sqrtf(ss)), epsr));
       if (st_piece < dpieces) {
         float* d = buf + row * ROWF + st_piece * NE;
 #pragma unroll
-        for (int q = 0; q < NE; q += 2) *(float2*)(d + q) = make_float2(e[q] / n, e[q + 1] / n);
+        for (int q = 0; q < NE; q += 2) *(float2*)(d + q) = make_float2(e[q] * rn, e[q + 1] * rn);
       }
     }
   };
@@ -213,9 +215,9 @@ __global__ __launch_bounds__(kThreads) void gram_kernel(GramArgs p) {
 #pragma unroll
         for (int q = 0; q < NE / 2; ++q) afrag[pc * (NE / 2) + q] = half ? e[2 * q + 1] : e[2 * q];
       }
-      const float n = fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr);
+      const float rn = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(__builtin_amdgcn_sqrtf(ss)), epsr));
 #pragma unroll
-      for (int s = 0; s < KS; ++s) afrag[s] = active ? afrag[s] / n : 0.f;
+      for (int s = 0; s < KS; ++s) afrag[s] = active ? afrag[s] * rn : 0.f;
     }
     float rsum[16], cval[16];
     int ccol[16];
