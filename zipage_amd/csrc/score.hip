@@ -107,13 +107,13 @@ template <> struct Rnd<BF16> {
 #ifdef ZP_DBG_NORND
     return;
 #endif
+    // v_cvt_pk_bf16_f32 with a zero in the low half: the 32-bit result IS the rounded value as
+    // fp32, so each value costs one instruction and nothing has to be unpacked
     typedef __attribute__((ext_vector_type(2))) float f2;
     typedef __attribute__((ext_vector_type(2))) __bf16 b2;
-    const f2 v = {a, b};
-    const b2 r = __builtin_convertvector(v, b2);
-    const uint32_t u = __builtin_bit_cast(uint32_t, r);
-    a = __uint_as_float(u << 16);
-    b = __uint_as_float(u & 0xffff0000u);
+    const f2 va = {0.f, a}, vb = {0.f, b};
+    a = __builtin_bit_cast(float, __builtin_convertvector(va, b2));
+    b = __builtin_bit_cast(float, __builtin_convertvector(vb, b2));
   }
 };
 template <> struct Rnd<F16> {
