@@ -73,6 +73,11 @@ def test_place_kv_pools_limits():
     made.clear()
     (k, v), rep = place_kv_pools(alloc, lambda a, b: 200.0, 16, span_bytes=50e9, pool_bytes=40e9)
     assert rep["slabs"] == 2                                             # always at least two pools
+    made.clear()
+    padded = []
+    (k, v), rep = place_kv_pools(alloc, lambda a, b: 200.0, 4, span_bytes=40e9, pool_bytes=1e9,
+                                 spacer=lambda n: padded.append(n))
+    assert rep["slabs"] == 4 and padded == [9e9] * 3                     # small pools step by span / slabs
 
 
 @pytest.mark.gpu

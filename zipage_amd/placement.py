@@ -62,19 +62,32 @@ def place_pools(alloc, probe, tries=6, good_enough=None):
     return best, {"tries": len(times), "probe_us": times, "kept": kept}
 
 
-def place_kv_pools(alloc_one, probe_pair, slabs=16, gain=0.93, span_bytes=160e9, pool_bytes=None):
+def place_kv_pools(alloc_one, probe_pair, slabs=16, gain=0.93, span_bytes=160e9, pool_bytes=None,
+                   spacer=None):
     """``alloc_one() -> pool`` allocates ONE pool-sized tensor; ``probe_pair(k, v) ->
     microseconds``.  Allocates pools side by side (all stay alive, so they cover consecutive
     regions of device memory) and probes the first one as the K pool against each new one as
     the V pool, until a pair runs in ``gain`` x the slowest pair's time or less (the new pool
-    reached another zone), ``slabs`` pools exist, their total passes ``span_bytes`` (needs
-    ``pool_bytes``) or memory runs out.  Returns ``((k, v), report)`` for the fastest pair; the
-    other pools are released."""
-    pools, times = [alloc_one()], {}
+    reached another zone), ``slabs`` pools exist, their span passes ``span_bytes`` (needs
+    ``pool_bytes``) or memory runs out.  Pools much smaller than ``span_bytes / slabs`` would
+    never leave the first zone, so ``spacer(nbytes)`` (default: a byte tensor on the pool's
+    device) pads each step to that size; spacers are released with the losing pools.  Returns
+    ``((k, v), report)`` for the fastest pair."""
+    pools, times, pads = [alloc_one()], {}, []
+    step = pool_bytes
+    if pool_bytes is not None and pool_bytes * max(2, slabs) < span_bytes:
+        step = span_bytes / max(2, slabs)
+        if spacer is None and isinstance(pools[0], torch.Tensor):
+            dev = pools[0].device
+            spacer = lambda n: torch.empty(int(n), dtype=torch.uint8, device=dev)
+        if spacer is None:
+            step = pool_bytes
     while len(pools) < max(2, slabs):
-        if pool_bytes is not None and len(pools) >= 2 and (len(pools) + 1) * pool_bytes > span_bytes:
+        if step is not None and len(pools) >= 2 and (len(pools) + 1) * step > span_bytes:
             break
         try:
+            if step is not None and step > pool_bytes:
+                pads.append(spacer(step - pool_bytes))
             pools.append(alloc_one())
         except torch.cuda.OutOfMemoryError:
             break
@@ -87,7 +100,7 @@ def place_kv_pools(alloc_one, probe_pair, slabs=16, gain=0.93, span_bytes=160e9,
     (ki, vi) = min(times, key=times.get)
     k, v = pools[ki], pools[vi]
     n = len(pools)
-    del pools
+    del pools, pads
     if torch.cuda.is_available():
         torch.cuda.empty_cache()
     return (k, v), {"slabs": n, "probe_us": {f"{i}-{j}": t for (i, j), t in times.items()},
