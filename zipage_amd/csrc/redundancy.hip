@@ -100,8 +100,9 @@ struct GramArgs {
   float threshold, eps;
 };
 
-template <typename T, bool RAW>
-__global__ __launch_bounds__(kThreads) void gram_kernel(GramArgs p) {
+template <typename T, bool RAW, int NW>
+__global__ __launch_bounds__(NW * 64) void gram_kernel(GramArgs p) {
+  constexpr int kThreads = NW * 64, kWaves = NW;    // shadow the file-wide 4-wave constants
   constexpr int NE = Unpack<T>::N;                  // elements per 16-byte piece
   constexpr int PIECES = kDmax / NE;                // pieces per full key row
   constexpr int ROWS_PER_IT = kThreads / PIECES;
@@ -1354,13 +1355,17 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
     else hipLaunchKernelGGL((gram_split_kernel<T, RAW, 4>), grid, dim3(kThreads), smem, st, a);
   } else {
     const size_t smem = sizeof(float) * 2 * TN * ROWF + tail;
+    // more row blocks than 4 waves: 8 waves take the page's rows in one pass, so every column
+    // tile is staged (and normalised) once instead of twice
+    const bool wide = a.BS / 32 > kWaves;
+    const void* fn = wide ? (const void*)gram_kernel<T, RAW, 8> : (const void*)gram_kernel<T, RAW, 4>;
     if (smem > 64 * 1024 &&
-        hipFuncSetAttribute((const void*)gram_kernel<T, RAW>,
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+        hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
       zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
       return ZP_EHIP;
     }
-    hipLaunchKernelGGL((gram_kernel<T, RAW>), grid, dim3(kThreads), smem, st, a);
+    if (wide) hipLaunchKernelGGL((gram_kernel<T, RAW, 8>), grid, dim3(512), smem, st, a);
+    else hipLaunchKernelGGL((gram_kernel<T, RAW, 4>), grid, dim3(kThreads), smem, st, a);
   }
   ZP_LAUNCH_CHECK();
   return ZP_OK;
