@@ -51,7 +51,8 @@ constexpr int kThreads = 256;
 constexpr int kWaves = 4;
 constexpr int kDmax = 128;
 constexpr int TN = 64;                  // keys per column tile
-constexpr int ROWF = kDmax + 2;         // floats per LDS row (bank-conflict-free pad)
+constexpr int ROWF = kDmax + 4;         // floats per LDS row: 16-byte aligned rows whose 16-byte reads by
+                                        // eight consecutive rows fall into eight different bank groups
 constexpr int KS = kDmax / 2;           // MFMA k-steps (2 per instruction)
 
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
@@ -199,7 +200,9 @@ __global__ __launch_bounds__(NW * 64) void gram_kernel(GramArgs p) {
   for (int rr = 0; rr < NR; ++rr) {
     const int rb = rr * kWaves + wave;
     const bool active = rb < row_blocks;
-    // ---- A fragments: this lane's key row, normalised; element k = 2s + half
+    // ---- A fragments: this lane's key row, normalised.  The order of the contraction index is
+    // free as long as both operands agree: k-step 4j + i of wave half `half` takes element
+    // 8j + 4 half + i, so a lane's B operands for four steps are one 16-byte LDS read.
     float afrag[KS];
     {
       const int slot = (active ? rb : 0) * 32 + col;
@@ -213,8 +216,19 @@ __global__ __launch_bounds__(NW * 64) void gram_kernel(GramArgs p) {
         Unpack<T>::run(v, e);
 #pragma unroll
         for (int q = 0; q < NE; ++q) ss += e[q] * e[q];
+        if constexpr (NE == 4) {
+          // piece pc holds elements 4 pc .. 4 pc + 3 = (j, half) = (pc / 2, pc % 2)
+          if ((pc & 1) == 0) {
 #pragma unroll
-        for (int q = 0; q < NE / 2; ++q) afrag[pc * (NE / 2) + q] = half ? e[2 * q + 1] : e[2 * q];
+            for (int q = 0; q < 4; ++q) afrag[(pc >> 1) * 4 + q] = e[q];
+          } else if (half) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) afrag[(pc >> 1) * 4 + q] = e[q];
+          }
+        } else {
+#pragma unroll
+          for (int q = 0; q < NE / 2; ++q) afrag[pc * (NE / 2) + q] = half ? e[2 * q + 1] : e[2 * q];
+        }
       }
       const float rn = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(__builtin_amdgcn_sqrtf(ss)), epsr));
 #pragma unroll
@@ -239,10 +253,22 @@ __global__ __launch_bounds__(NW * 64) void gram_kernel(GramArgs p) {
           f32x16_t acc;
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-          const float* brow = cur + (st * 32 + col) * ROWF + half;
+          if constexpr (NE == 4) {
+            const float4* b4 = (const float4*)(cur + (st * 32 + col) * ROWF + 4 * half);
 #pragma unroll
-          for (int s = 0; s < KS; ++s)
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[s], brow[2 * s], acc, 0, 0, 0);
+            for (int j4 = 0; j4 < KS / 4; ++j4) {
+              const float4 bv = b4[2 * j4];
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 0], bv.x, acc, 0, 0, 0);
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 1], bv.y, acc, 0, 0, 0);
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 2], bv.z, acc, 0, 0, 0);
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 3], bv.w, acc, 0, 0, 0);
+            }
+          } else {
+            const float* brow = cur + (st * 32 + col) * ROWF + half;
+#pragma unroll
+            for (int s = 0; s < KS; ++s)
+              acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[s], brow[2 * s], acc, 0, 0, 0);
+          }
           const int cslot = toff + st * 32 + col;
           const int cidx = jc * p.BS + cslot;  // logical column index of this lane
           const bool same_page = jc == jp;
