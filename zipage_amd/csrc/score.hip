@@ -68,7 +68,7 @@ template <> struct Mma<F16> {
 };
 template <> struct Mma<F32> {
   typedef float Frag;
-  static constexpr int KPI = 2, EPL = 1, KS = kDmax / KPI, TN = 16 * kWaves, ROWB = kDmax * 4 + 8;
+  static constexpr int KPI = 2, EPL = 1, KS = kDmax / KPI, TN = 16 * kWaves, ROWB = kDmax * 4 + 16;
   __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
   }
@@ -272,7 +272,10 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
                                 ((int64_t)a_w * p.Hq + (int64_t)h * p.G + a_g) * p.D) * T::bytes;
 #pragma unroll
       for (int s = 0; s < KS; ++s) {
-        const int k0 = s * M::KPI + half * M::EPL;
+        // fp32: the order of the contraction index is free as long as both operands agree;
+        // k-step 4j + i of wave half `half` takes element 8j + 4 half + i, so that a lane's B
+        // operands for four steps are one 16-byte LDS read
+        const int k0 = T::bytes == 4 ? 8 * (s >> 2) + 4 * half + (s & 3) : s * M::KPI + half * M::EPL;
         if (a_ok && k0 < p.D) afrag[s] = *(const Frag*)(qrow + (int64_t)k0 * T::bytes);
         else zero_frag<T>(afrag[s]);
       }
@@ -338,13 +341,23 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[r] = 0.f;
             const char* brow = cur + (st * 32 + col) * ROWB + half * M::EPL * T::bytes;
+            const char* brow4 = cur + (st * 32 + col) * ROWB + half * 16;   // fp32 operand order
             // all B fragments of the subtile are requested before the first MFMA needs one
             constexpr int KB = KS < 8 ? KS : 8;
 #pragma unroll
             for (int s0 = 0; s0 < KS; s0 += KB) {
               Frag bfr[KB];
 #pragma unroll
-              for (int s = 0; s < KB; ++s) bfr[s] = *(const Frag*)(brow + (s0 + s) * M::KPI * T::bytes);
+              for (int s = 0; s < KB; ++s) {
+                if constexpr (T::bytes == 4) {
+                  if ((s & 3) == 0) {
+                    const float4 b4 = *(const float4*)(brow4 + ((s0 + s) >> 2) * 32);
+                    __builtin_memcpy(&bfr[s], &b4, 16);
+                  }
+                } else {
+                  bfr[s] = *(const Frag*)(brow + (s0 + s) * M::KPI * T::bytes);
+                }
+              }
               __builtin_amdgcn_sched_barrier(0);  // keep the reads grouped ahead of the MFMAs
 #pragma unroll
               for (int s = 0; s < KB; ++s) acc = M::mma(afrag[s0 + s], bfr[s], acc);
