@@ -47,6 +47,15 @@ __device__ __forceinline__ void last_claim_reduce(int& c, float& v) {
 #undef ZP_CLAIM_STEP
 }
 
+// A similarity as 2^-32 fixed point (two's complement in an unsigned 64-bit word) and back: sums of
+// such words are exact and independent of the order of the additions.
+__device__ __forceinline__ unsigned long long to_fixed32(float v) {
+  return (unsigned long long)(long long)(v * 4294967296.f);
+}
+__device__ __forceinline__ float from_fixed32(unsigned long long w) {
+  return (float)(long long)w * (1.f / 4294967296.f);
+}
+
 constexpr int kThreads = 256;
 constexpr int kWaves = 4;
 constexpr int kDmax = 128;
@@ -113,7 +122,8 @@ __global__ __launch_bounds__(NW * 64) void gram_kernel(GramArgs p) {
   extern __shared__ __align__(16) char smem[];
   float* kbuf0 = (float*)smem;
   float* kbuf1 = kbuf0 + TN * ROWF;
-  float* l_sum = kbuf1 + TN * ROWF;                 // lightning: [BS] row sums
+  unsigned long long* l_corr = (unsigned long long*)(kbuf1 + TN * ROWF);   // lightning: [BS] claimed from a row
+  float* l_sum = (float*)(l_corr + (RAW ? 0 : p.BS));                     //            [BS] row sums
   float* l_val = l_sum + (RAW ? 0 : p.BS);          //            [BS] claimed values
   int* l_col = (int*)(l_val + (RAW ? 0 : p.BS));    //            [BS] claimed columns
   int* vpage = l_col + (RAW ? 0 : p.BS);            // [NB] valid page ids (raw)
@@ -309,13 +319,18 @@ __global__ __launch_bounds__(NW * 64) void gram_kernel(GramArgs p) {
     }
   }
   if (!RAW) {
+    // every key hands the value of its claimed entry to the row it was taken from; several keys
+    // may claim from one row, so the values are added as 2^-32 fixed point: exact to 2^-33 per
+    // term and independent of the order (a scan of all keys per row cost ~10 % of the kernel)
+    for (int i = tid; i < p.BS; i += kThreads) l_corr[i] = 0ull;
     __syncthreads();
-    for (int i = tid; i < p.BS; i += kThreads) {
-      float corr = 0.f;
-      for (int j = 0; j < p.BS; ++j)
-        if (l_col[j] == i) corr += l_val[j];
-      Elem<T>::st(p.r_out, orow * Tn + (int64_t)jp * p.BS + i, l_sum[i] - corr);
+    for (int j = tid; j < p.BS; j += kThreads) {
+      const int c = l_col[j];
+      if (c >= 0 && c < p.BS) atomicAdd(&l_corr[c], to_fixed32(l_val[j]));
     }
+    __syncthreads();
+    for (int i = tid; i < p.BS; i += kThreads)
+      Elem<T>::st(p.r_out, orow * Tn + (int64_t)jp * p.BS + i, l_sum[i] - from_fixed32(l_corr[i]));
   }
 }
 
@@ -583,14 +598,6 @@ __device__ __forceinline__ void split8_pk(const float* x, u32x4& hi, u32x4& lo) 
   }
 }
 
-// A similarity as 2^-32 fixed point (two's complement in an unsigned 64-bit word) and back: sums of
-// such words are exact and independent of the order of the additions.
-__device__ __forceinline__ unsigned long long to_fixed32(float v) {
-  return (unsigned long long)(long long)(v * 4294967296.f);
-}
-__device__ __forceinline__ float from_fixed32(unsigned long long w) {
-  return (float)(long long)w * (1.f / 4294967296.f);
-}
 
 // Largest value over the 32 lanes of a wave half.
 __device__ __forceinline__ int half_max_i(int v) {
@@ -1334,7 +1341,7 @@ int check_common(const char* name, const void* k_cache, const int32_t* table, vo
 template <typename T, bool RAW>
 int launch_gram(const GramArgs& a, int L, hipStream_t st) {
   dim3 grid((unsigned)((int64_t)L * a.B * a.Hkv * a.NB));
-  const size_t tail = (RAW ? 0 : (size_t)a.BS * 12) + sizeof(int) * 2 * a.NB;
+  const size_t tail = (RAW ? 0 : (size_t)a.BS * 20) + sizeof(int) * 2 * a.NB;
   if constexpr (T::bytes == 2 && !RAW) {
     if (a.BS <= kPageRows && a.BS % 32 == 0) {
       const size_t smem = (size_t)kPageRows * ROWH + (size_t)kPageRows * 20 +
