@@ -368,7 +368,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gram_split_kernel(Gr
   extern __shared__ __align__(16) char smem[];
   char* buf0 = smem;                                // [hi plane][lo plane]
   char* buf1 = smem + 2 * PLANE;
-  float* l_sum = (float*)(smem + 4 * PLANE);
+  unsigned long long* l_corr = (unsigned long long*)(smem + 4 * PLANE);   // [BS] claimed from a row
+  float* l_sum = (float*)(l_corr + (RAW ? 0 : p.BS));
   float* l_val = l_sum + (RAW ? 0 : p.BS);
   int* l_col = (int*)(l_val + (RAW ? 0 : p.BS));
   int* vpage = l_col + (RAW ? 0 : p.BS);
@@ -556,13 +557,17 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gram_split_kernel(Gr
     }
   }
   if (!RAW) {
+    // claim values go to the rows they were taken from as 2^-32 fixed-point atomics
+    // (order-independent), not through a scan of all claims per row
+    for (int i = tid; i < p.BS; i += kThreads) l_corr[i] = 0ull;
     __syncthreads();
-    for (int i = tid; i < p.BS; i += kThreads) {
-      float corr = 0.f;
-      for (int j = 0; j < p.BS; ++j)
-        if (l_col[j] == i) corr += l_val[j];
-      Elem<T>::st(p.r_out, orow * Tn + (int64_t)jp * p.BS + i, l_sum[i] - corr);
+    for (int j = tid; j < p.BS; j += kThreads) {
+      const int c = l_col[j];
+      if (c >= 0 && c < p.BS) atomicAdd(&l_corr[c], to_fixed32(l_val[j]));
     }
+    __syncthreads();
+    for (int i = tid; i < p.BS; i += kThreads)
+      Elem<T>::st(p.r_out, orow * Tn + (int64_t)jp * p.BS + i, l_sum[i] - from_fixed32(l_corr[i]));
   }
 }
 
