@@ -39,12 +39,19 @@ struct F32  { typedef float raw;    static constexpr int bytes = 4; };
 __device__ __forceinline__ float bf16_bits_to_float(uint16_t h) {
   return __uint_as_float(((uint32_t)h) << 16);
 }
-// Round-to-nearest-even, infinities preserved, NaN kept quiet.
+// Round-to-nearest-even, infinities preserved, NaN kept quiet: the hardware conversion
+// (v_cvt_pk_bf16_f32), one instruction.
+typedef float zp_f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 zp_bf16x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
+  const zp_f32x2 v = {f, 0.f};
+  return (uint16_t)__builtin_bit_cast(uint32_t, __builtin_convertvector(v, zp_bf16x2));
+}
+// The rounded value as fp32: with the value in the high half of the packed result and a zero in
+// the low half, the 32-bit result is the answer.
+__device__ __forceinline__ float bf16_round(float f) {
+  const zp_f32x2 v = {0.f, f};
+  return __builtin_bit_cast(float, __builtin_convertvector(v, zp_bf16x2));
 }
 __device__ __forceinline__ float f16_bits_to_float(uint16_t h) {
   union { uint16_t u; _Float16 f; } c; c.u = h; return (float)c.f;
@@ -57,7 +64,7 @@ template <typename T> struct Elem;
 template <> struct Elem<BF16> {
   __device__ static __forceinline__ float ld(const void* p, int64_t i) { return bf16_bits_to_float(((const uint16_t*)p)[i]); }
   __device__ static __forceinline__ void st(void* p, int64_t i, float v) { ((uint16_t*)p)[i] = float_to_bf16_bits(v); }
-  __device__ static __forceinline__ float rnd(float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); }
+  __device__ static __forceinline__ float rnd(float v) { return bf16_round(v); }
 };
 template <> struct Elem<F16> {
   __device__ static __forceinline__ float ld(const void* p, int64_t i) { return f16_bits_to_float(((const uint16_t*)p)[i]); }
