@@ -12,6 +12,8 @@
 //   gram_kernel        fp32 caches, both variants: v_mfma_f32_32x32x2_f32 on keys divided by
 //                      their cache-dtype norm in fp32 (the reference's arithmetic), full
 //                      matrix, a wave owns 32 rows for all columns.
+//   gram_page_f32_kernel  fp32 caches, lightning, pages of at most 256 keys: the normalised page
+//                      resident in LDS, one barrier, both operands read from that copy.
 //   gram_split_kernel  16-bit caches, lightning with pages above 256 keys: normalised keys
 //                      split into two bf16 planes, three MFMAs per k-step, full matrix.
 //   gram_page_kernel   16-bit caches, lightning: stored keys on the matrix cores, 1/norm
@@ -332,6 +334,134 @@ __global__ __launch_bounds__(NW * 64) void gram_kernel(GramArgs p) {
     for (int i = tid; i < p.BS; i += kThreads)
       Elem<T>::st(p.r_out, orow * Tn + (int64_t)jp * p.BS + i, l_sum[i] - from_fixed32(l_corr[i]));
   }
+}
+
+// ------------------------------------------------------------------ fp32 caches, lightning, whole page in LDS
+// One workgroup per (layer, sequence, head, page) of at most 256 keys: the page is loaded once
+// with coalesced 16-byte loads, normalised on the way into LDS (132 KB), and after ONE barrier
+// every wave multiplies its 32 rows (A operand read from the same LDS copy) with all column
+// blocks: no tile pipeline, no further barriers, no strided per-lane row loads.
+constexpr int kPage32Rows = 256;
+constexpr int kPage32Threads = 512;
+__global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs p) {
+  typedef F32 T;
+  constexpr int PIECES = kDmax / 4;                            // 16-byte pieces per key row (32)
+  constexpr int ROWS_PER_IT = kPage32Threads / PIECES;         // 16
+  constexpr int ITERS = kPage32Rows / ROWS_PER_IT;             // 16
+  extern __shared__ __align__(16) char smem[];
+  float* kpl = (float*)smem;                                   // [256][ROWF] normalised keys
+  unsigned long long* l_corr = (unsigned long long*)(kpl + kPage32Rows * ROWF);
+  float* l_sum = (float*)(l_corr + kPage32Rows);
+  float* l_val = l_sum + kPage32Rows;
+  int* l_col = (int*)(l_val + kPage32Rows);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const int jp = blockIdx.x % p.NB;
+  const int h = (blockIdx.x / p.NB) % p.Hkv;
+  const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
+  const int l = blockIdx.x / (p.NB * p.Hkv * p.B);
+  const int Tn = p.NB * p.BS;
+  const int64_t obase = (((int64_t)l * p.B + b) * p.Hkv + h) * Tn + (int64_t)jp * p.BS;
+
+  const int code = p.table[(int64_t)b * p.NB + jp];
+  int rpid = page_is_pad(code) ? -1 : page_id(code);
+  if (rpid >= p.num_pages) rpid = -1;
+  if (rpid < 0) {
+    for (int s = tid; s < p.BS; s += kPage32Threads) Elem<T>::st(p.r_out, obase + s, -INFINITY);
+    return;
+  }
+  const int dpieces = p.D / 4;
+  const int64_t k_row = (int64_t)p.Hkv * p.D * 4;
+  const char* page = p.k + (l * p.k_sl + (int64_t)rpid * p.k_sp) * 4 + (int64_t)h * p.D * 4;
+
+  // ---- stage: all loads of the page in flight, then norms and the normalised copy
+  {
+    const int piece = tid % PIECES, row0 = tid / PIECES;
+    float4 raw[ITERS];
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int row = it * ROWS_PER_IT + row0;
+      raw[it] = *(const float4*)(page + (int64_t)(row < p.BS ? row : 0) * k_row +
+                                 (piece < dpieces ? piece : 0) * 16);
+    }
+    if (tid < kPage32Rows) l_corr[tid] = 0ull;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const int row = it * ROWS_PER_IT + row0;
+      if (!(row < p.BS && piece < dpieces)) raw[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+      const float4 e = raw[it];
+      float ss = (e.x * e.x + e.y * e.y) + (e.z * e.z + e.w * e.w);
+      ss = pieces_sum<PIECES>(ss);
+      const float rn = __builtin_amdgcn_rcpf(fmaxf(__builtin_amdgcn_sqrtf(ss), p.eps));
+      *(float4*)(kpl + row * ROWF + piece * 4) = make_float4(e.x * rn, e.y * rn, e.z * rn, e.w * rn);
+    }
+  }
+  __syncthreads();
+
+  const int nrb = p.BS / 32;
+  if (wave < nrb) {
+    const int rb = wave;
+    float afrag[KS];
+    {
+      const float4* a4 = (const float4*)(kpl + (rb * 32 + col) * ROWF + 4 * half);
+#pragma unroll
+      for (int j4 = 0; j4 < KS / 4; ++j4) {
+        const float4 av = a4[2 * j4];
+        afrag[4 * j4 + 0] = av.x; afrag[4 * j4 + 1] = av.y;
+        afrag[4 * j4 + 2] = av.z; afrag[4 * j4 + 3] = av.w;
+      }
+    }
+    float rsum[16], cval[16];
+    int ccol[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { rsum[r] = 0.f; cval[r] = 0.f; ccol[r] = -1; }
+#pragma unroll 1
+    for (int cb = 0; cb < nrb; ++cb) {
+      f32x16_t acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+      const float4* b4 = (const float4*)(kpl + (cb * 32 + col) * ROWF + 4 * half);
+#pragma unroll
+      for (int j4 = 0; j4 < KS / 4; ++j4) {
+        const float4 bv = b4[2 * j4];
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 0], bv.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 1], bv.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 2], bv.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 3], bv.w, acc, 0, 0, 0);
+      }
+      const int cslot = cb * 32 + col;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+        float sv = acc[r];
+        if (rslot == cslot) sv = 0.f;
+        rsum[r] += sv;
+        if (sv > p.threshold) { ccol[r] = cslot; cval[r] = sv; }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float sv = half_sum(rsum[r]);
+      int c = ccol[r];
+      float v = cval[r];
+      last_claim_reduce(c, v);
+      if (col == 0) {
+        const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+        l_sum[rslot] = sv;
+        l_col[rslot] = c;
+        l_val[rslot] = v;
+      }
+    }
+  }
+  __syncthreads();
+  for (int j = tid; j < p.BS; j += kPage32Threads) {
+    const int c = l_col[j];
+    if (c >= 0 && c < p.BS) atomicAdd(&l_corr[c], to_fixed32(l_val[j]));
+  }
+  __syncthreads();
+  for (int i = tid; i < p.BS; i += kPage32Threads)
+    Elem<T>::st(p.r_out, obase + i, l_sum[i] - from_fixed32(l_corr[i]));
 }
 
 // ------------------------------------------------------------------ 16-bit caches: split-bf16 Gram
@@ -1357,6 +1487,19 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
         return ZP_EHIP;
       }
       hipLaunchKernelGGL((gram_page_kernel<T>), grid, dim3(kPageThreads), smem, st, a);
+      ZP_LAUNCH_CHECK();
+      return ZP_OK;
+    }
+  }
+  if constexpr (T::bytes == 4 && !RAW) {
+    if (a.BS <= kPage32Rows && a.BS % 32 == 0) {
+      const size_t smem = (size_t)kPage32Rows * ROWF * 4 + (size_t)kPage32Rows * 20;
+      if (hipFuncSetAttribute((const void*)gram_page_f32_kernel,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+        zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
+        return ZP_EHIP;
+      }
+      hipLaunchKernelGGL(gram_page_f32_kernel, grid, dim3(kPage32Threads), smem, st, a);
       ZP_LAUNCH_CHECK();
       return ZP_OK;
     }
