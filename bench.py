@@ -4,11 +4,15 @@
 A step is one pass of the compression pipeline (score -> max-pool 7 -> window mask ->
 top-2048 per kv head -> in-place compaction to 8 pages) over one batch of synthetic ragged
 sequences at Qwen3-8B attention shape (32 q heads, 8 kv heads, head_dim 128, bf16, page 256,
-window 32), one layer, inputs resident in HBM.  Prints ONE JSON line.
+window 32), inputs resident in HBM.  The default workload is the one the metric is quoted on,
+BASELINE configs[3]: 256 ragged sequences of 9-10 pages, groups of 16 sharing two prefix pages
+(copy-on-write targets), all 36 layers per step (one layer at a time over one page pool).
+Prints ONE JSON line.
 
-After it, unless --no-e2e, the same process runs BASELINE's end-to-end case (random-init
-Qwen3-8B, 256 requests x 512-token prompts x 4096 greedy tokens, budget 8 pages) through the
-decode engine and adds decode tokens/s and the compression share as `end_to_end`.
+After it, unless --no-extra-legs, the same process adds the 64-sequence single-layer workload
+(BASELINE configs[1]) as `configs1_b64`, and, unless --no-e2e, BASELINE's end-to-end case
+(random-init Qwen3-8B, 256 requests x 512-token prompts x 4096 greedy tokens, budget 8 pages)
+through the decode engine as `end_to_end` (decode tokens/s and the compression share).
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--no-cpu-baseline] [--no-e2e]
   python bench.py --config 5 [--requests R] [--prompt P] [--out-tokens T] [--sync-compress]
@@ -26,14 +30,20 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes one compaction launch moves per (sequence, layer), from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE scaled by a plain copy kernel (profiles/pipeline_cfg2_b64.md)
-COMPACT_TRAFFIC_PER_SEQ_LAYER = 16_803_258
+# HBM bytes one compaction launch moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# program on the named workload, scaled by a plain copy kernel of known size (--calibrate-copy).
+# Counters cannot be read from inside the benchmark, so these are figures of earlier profiled runs
+# of the same workload (keyed by config and batch); --traffic overrides them, and a workload
+# without a counter run reports null.
+COMPACT_TRAFFIC = {
+    (2, 64): (1_075_408_512, "profiles/pipeline_cfg2_b64.md"),
+}
 
 
-def cpu_baseline(wl, cfg, sample_seqs, budget_s=30.0):
+def cpu_baseline(wl, cfg, sample_seqs, layers=1, budget_s=30.0):
     """The CPU oracle (a PyTorch port of the reference algorithm) on the first
-    ``sample_seqs`` sequences of the same workload, on the host cores."""
+    ``sample_seqs`` sequences of the same workload, one layer, on the host cores; a workload of
+    ``layers`` layers is reported as that time x ``layers``."""
     import torch
     from oracle import zipage_oracle as O
     cores = os.cpu_count() or 1
@@ -57,9 +67,11 @@ def cpu_baseline(wl, cfg, sample_seqs, budget_s=30.0):
             break
     times.sort()
     med = times[len(times) // 2]
-    return {"value": b / med, "unit": "sequences/s (one layer)", "cores": cores, "kind": "port",
+    unit = "sequences/s (one layer)" if layers == 1 else f"sequences/s ({layers} layers)"
+    return {"value": b / (med * layers), "unit": unit, "cores": cores, "kind": "port",
             "sample": f"first {b} sequences of the same batch, 1 layer, median of {len(times)} runs "
-                      f"after 1 warm-up ({med * 1e3:.0f} ms per run)"}
+                      f"after 1 warm-up ({med * 1e3:.0f} ms per run)"
+                      + ("" if layers == 1 else f"; the figure is that time x {layers} layers")}
 
 
 def end_to_end(requests=256, prompt=512, out_tokens=4096, async_compress=True, ragged=False,
@@ -131,86 +143,18 @@ def end_to_end(requests=256, prompt=512, out_tokens=4096, async_compress=True, r
     return out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--batch", type=int, default=None)
-    ap.add_argument("--config", type=int, default=2, choices=[2, 3, 4, 5],
-                    help="workload, numbered from 1 as in BASELINE.json: 2 = 64 ragged sequences, one "
-                         "layer (default, the headline line); 3 = 128 sequences at Qwen3-0.6B "
-                         "shape in fp32 with the global-score and redundancy terms (lightning; "
-                         "--pipeline-switches raw for all pairs); 4 = 256 sequences with shared "
-                         "prefixes and copy-on-write targets, 36 layers run one layer at a time "
-                         "over one page pool; 5 = the end-to-end decode case alone")
-    ap.add_argument("--no-e2e", action="store_true",
-                    help="skip the end-to-end decode leg that follows the default run")
-    ap.add_argument("--requests", type=int, default=256)
-    ap.add_argument("--prompt", type=int, default=512)
-    ap.add_argument("--out-tokens", type=int, default=4096)
-    ap.add_argument("--sync-compress", action="store_true",
-                    help="end-to-end leg: compress in line with the decode steps instead of on "
-                         "the side stream")
-    ap.add_argument("--script-switches", action="store_true",
-                    help="end-to-end leg: compress with the switch set of the reference's scripts "
-                         "(global score, lightning redundancy, pooling) instead of pooling alone")
-    ap.add_argument("--pipeline-switches", choices=["pooling", "scripts", "raw"], default="pooling",
-                    help="compression switches of the single-layer leg: pooling alone (default, the "
-                         "headline line), the reference scripts' set (window 16, global score, "
-                         "lightning redundancy, pooling 5) or raw all-pairs redundancy with pooling 7; "
-                         "the non-default sets say so in config.workload")
-    ap.add_argument("--ragged-prompts", action="store_true",
-                    help="end-to-end leg: prompt lengths uniform in [P/2, 3P/2] so sequences reach "
-                         "their budget on different steps")
-    ap.add_argument("--separate-select-stages", action="store_true",
-                    help="run pooling, the mask epilogue and top-k as three launches (timed under "
-                         "the reference's stage names) instead of the one-launch selection")
-    ap.add_argument("--place-tries", type=int, default=16,
-                    help="most pool-sized allocations made side by side before any data is written "
-                         "(allocation stops as soon as a pair is fast or 160 GB are held); a small "
-                         "timed gather on pairs of them picks the K pool and the V pool (the "
-                         "in-place compaction is ~15 %% faster when the two lie in different regions "
-                         "of device memory; an engine allocates its pools once and can do the "
-                         "same); every probe figure is reported in 'placement'; 1 = take the first "
-                         "two allocations")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--cpu-sample", type=int, default=64)
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run a plain 1 GiB device copy (read 1 GiB, write 1 GiB) so that a "
-                         "rocprofv3 --pmc run of this command has a kernel of known traffic to "
-                         "scale FETCH_SIZE / WRITE_SIZE by")
-    ap.add_argument("--traffic", type=float, default=None,
-                    help="HBM bytes per compaction launch measured with rocprofv3 --pmc "
-                         "(reported as roofline.traffic)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build measures the single-GPU hot path only; run with --gpus 1 "
-              "(every (sequence, kv head, layer) is independent, so more GPUs shard sequences "
-              "with no exchange step).", file=sys.stderr)
-        sys.exit(2)
-
+def run_pipeline(config, args, sw="pooling", batch=None, steps=None, warmup=None):
+    """One compression workload (numbered from 1 as in BASELINE.json): build it in HBM, run
+    ``warmup`` untimed and ``steps`` timed steps, then a second pass with events around every
+    stage.  Returns the JSON-ready dict of the run (without the contract's fixed keys)."""
     import torch
-    from zipage_amd import _lib
     from zipage_amd.compress import CompressConfig, StageTimer, compress_layers
     from zipage_amd.workload import algorithmic_bytes, ragged_batch
 
-    _lib.load()  # fail loudly if the HIP library is missing
-    torch.cuda.set_device(0)
-    if args.config == 5:
-        e2e = end_to_end(args.requests, args.prompt, args.out_tokens, not args.sync_compress,
-                         args.ragged_prompts, args.script_switches)
-        print(json.dumps({
-            "metric": "decode tokens/sec", "value": e2e["decode_tok_per_s"], "unit": "tokens/s",
-            "n_gpus": 1, "steps": e2e["decode_steps"], "warmup": 0,
-            "ms_per_step": e2e["ms_per_decode_step"], "higher_is_better": True, "scaling": "weak",
-            "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-            "config": {"workload": e2e["workload"]}, "roofline": e2e["decode_attention"],
-            "cpu_baseline": None, "end_to_end": e2e}))
-        return
-    sw = args.pipeline_switches
-    if args.config == 2:
-        batch, layers = args.batch or 64, 1
+    steps = args.steps if steps is None else steps
+    warmup = args.warmup if warmup is None else warmup
+    if config == 2:
+        batch, layers = batch or 64, 1
         wl = ragged_batch(batch, L=1, pool_pages=20000, budget=8, W=16 if sw == "scripts" else 32,
                           seed=1, lengths=(2049, 2304), name="cfg2",
                           with_score_cache=sw == "scripts", compressed=sw == "scripts",
@@ -218,9 +162,9 @@ def main():
         desc = (f"configs[1]: {batch} ragged sequences, 1 layer, Qwen3-8B attention shape (32q/8kv "
                 "heads, head_dim 128), bf16, 9 pages x 256 tokens, window 32, 20k-page pool, score "
                 "-> max-pool 7 -> top-2048/head -> compact to 8 pages")
-    elif args.config == 3:
+    elif config == 3:
         from zipage_amd.workload import QWEN3_0_6B
-        batch, layers = args.batch or 128, 1
+        batch, layers = batch or 128, 1
         wl = ragged_batch(batch, L=1, pool_pages=2048, budget=8, W=32, seed=0, lengths=(2304, 2304),
                           dtype=torch.float32, shape=QWEN3_0_6B, name="cfg3", with_score_cache=True,
                           compressed=True, place_tries=args.place_tries)
@@ -230,15 +174,17 @@ def main():
                 + ("raw all-pairs" if sw == "raw" else "lightning (same-page)")
                 + " redundancy (lambda 2/3) -> top-2048/head -> compact to 8 pages")
     else:
-        batch, layers = args.batch or 256, 36
+        batch, layers = batch or 256, 36
         wl = ragged_batch(batch, L=1, pool_pages=60000, budget=8, W=32, seed=3,
                           lengths=(2049, 2560), shared_prefix_group=16, shared_prefix_pages=2,
                           name="cfg4", place_tries=args.place_tries)
-        desc = (f"configs[3]: {batch} ragged sequences (9-10 pages), groups of 16 share 2 prefix "
-                "pages (copy-on-write targets), 60k-page pool, Qwen3-8B shape, bf16, 36 layers run "
-                "one layer at a time over the same pool")
+        desc = (f"configs[3]: {batch} ragged sequences (9-10 pages x 256 tokens), groups of 16 share "
+                "2 prefix pages (copy-on-write targets), 60k-page pool, Qwen3-8B attention shape "
+                "(32q/8kv heads, head_dim 128), bf16, window 32, score -> max-pool 7 -> "
+                "top-2048/head -> compact to 8 pages, 36 layers per step run one layer at a time "
+                "over the same pool")
     cfg = CompressConfig(budget_blocks=8, query_cache_len=32, enable_pooling=True, pooling_size=7)
-    if args.config == 3:
+    if config == 3:
         if sw == "scripts":
             sys.exit("bench.py: --config 3 takes --pipeline-switches pooling (lightning) or raw")
         cfg = CompressConfig(budget_blocks=8, query_cache_len=32, use_global_score=True,
@@ -247,7 +193,7 @@ def main():
                              enable_pooling=True, continues_pooling=True, pooling_size=7,
                              pooling_mode="avg")
     elif sw != "pooling":
-        if args.config != 2:
+        if config != 2:
             sys.exit("bench.py: --pipeline-switches applies to --config 2 and 3")
         if sw == "scripts":
             cfg = CompressConfig(budget_blocks=8, query_cache_len=16, use_global_score=True,
@@ -266,6 +212,159 @@ def main():
                             wl.compressed, wl.targets, cfg, timer=timer,
                             fused_select=not args.separate_select_stages)
 
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    # timed region: only the roofline kernel carries events (each event pair costs the stream a
+    # few microseconds, 8 % of a step when every stage has one)
+    kv_timer = StageTimer(True, only=("compress_kv",))
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step(kv_timer)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    # the per-stage breakdown comes from a second, untimed pass with events around every stage
+    timer = StageTimer(True)
+    for _ in range(min(steps, max(1, 200 // layers))):
+        step(timer)
+    torch.cuda.synchronize()
+    stage_steps = min(steps, max(1, 200 // layers))
+
+    stage_s = timer.seconds()
+    ms_per_step = elapsed / steps * 1e3
+    seqs_per_s = wl.B / (elapsed / steps)
+    alg = algorithmic_bytes(wl, cfg)  # one layer
+    kv_s = kv_timer.seconds()["compress_kv"] / (steps * layers)
+    achieved = alg["compress_kv"] / kv_s / 1e9
+    stages_ms = {k: round(v / (stage_steps * layers) * 1e3, 4) for k, v in stage_s.items()}
+    gpu_ms = sum(stage_s.values()) / (stage_steps * layers) * 1e3  # per layer
+    if args.traffic is not None:
+        traffic, traffic_src = args.traffic, "--traffic"
+    elif (config, wl.B) in COMPACT_TRAFFIC and sw == "pooling":
+        traffic, traffic_src = COMPACT_TRAFFIC[(config, wl.B)]
+        traffic_src = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this workload, "
+                       "scaled by the calibration copy: " + traffic_src)
+    else:
+        traffic, traffic_src = None, "no counter run of this workload"
+    roof = {"bound": "hbm", "kernel": "compact_kernel (compress_kv)",
+            "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": traffic, "traffic_source": traffic_src,
+            "algorithmic_bytes": alg["compress_kv"],
+            "avg_launch_us": round(kv_s * 1e6, 2)}
+    out = {
+        "value": round(seqs_per_s, 1),
+        "unit": "sequences/s (one layer)" if layers == 1 else f"sequences/s ({layers} layers)",
+        "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 4),
+        "dtype": "f32" if config == 3 else "bf16",
+        "config": {"workload": desc, "batch": wl.B, "layers": layers},
+        "roofline": roof,
+        "pipeline": {"algorithmic_bytes": alg["pipeline"],
+                     "gpu_ms_sum_of_stages_per_layer": round(gpu_ms, 4),
+                     "wall_ms_per_layer": round(ms_per_step / layers, 4),
+                     "hbm_frac_of_stage_time": round(alg["pipeline"] / (gpu_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "stages_ms": stages_ms},
+    }
+    if wl.placement is not None:
+        # the K / V pools were chosen among pool-sized allocations by a timed compaction of this
+        # batch (random keep flags); pair 0-1 is what the first two allocations give, and the
+        # engine's single cache allocation does not run this search: bench-only
+        out["placement"] = dict(wl.placement, scope="bench-only: the engine makes one cache allocation")
+        first = wl.placement["probe_us"].get("0-1")
+        if first:
+            roof["first_two_allocations"] = {
+                "avg_launch_us": first, "achieved": round(alg["compress_kv"] / first / 1e3, 1),
+                "frac": round(alg["compress_kv"] / first / 1e3 / HBM_PEAK_GBS, 4),
+                "note": "same kernel and batch with K and V in the first two pool allocations "
+                        "(probe before any data is written, 8 launches)"}
+        roof["placed"] = {"pools": wl.placement["kept"], "frac": roof["frac"]}
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(wl, cfg, min(args.cpu_sample, 16) if config == 3
+                                           else args.cpu_sample, layers)
+    del wl
+    torch.cuda.empty_cache()
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batch", type=int, default=None)
+    ap.add_argument("--config", type=int, default=4, choices=[2, 3, 4, 5],
+                    help="workload, numbered from 1 as in BASELINE.json: 4 (default, the headline "
+                         "line) = 256 ragged sequences with shared prefixes and copy-on-write "
+                         "targets, 36 layers per step run one layer at a time over one page pool; "
+                         "2 = 64 ragged sequences, one layer; 3 = 128 sequences at Qwen3-0.6B "
+                         "shape in fp32 with the global-score and redundancy terms (lightning; "
+                         "--pipeline-switches raw for all pairs); 5 = the end-to-end decode case "
+                         "alone")
+    ap.add_argument("--no-e2e", action="store_true",
+                    help="skip the end-to-end decode leg that follows the default run")
+    ap.add_argument("--no-extra-legs", action="store_true",
+                    help="skip the 64-sequence leg and the end-to-end leg that follow the default run")
+    ap.add_argument("--requests", type=int, default=256)
+    ap.add_argument("--prompt", type=int, default=512)
+    ap.add_argument("--out-tokens", type=int, default=4096)
+    ap.add_argument("--sync-compress", action="store_true",
+                    help="end-to-end leg: compress in line with the decode steps instead of on "
+                         "the side stream")
+    ap.add_argument("--script-switches", action="store_true",
+                    help="end-to-end leg: compress with the switch set of the reference's scripts "
+                         "(global score, lightning redundancy, pooling) instead of pooling alone")
+    ap.add_argument("--pipeline-switches", choices=["pooling", "scripts", "raw"], default="pooling",
+                    help="compression switches of --config 2 / 3: pooling alone (default), the "
+                         "reference scripts' set (window 16, global score, lightning redundancy, "
+                         "pooling 5) or raw all-pairs redundancy with pooling 7; the non-default "
+                         "sets say so in config.workload")
+    ap.add_argument("--ragged-prompts", action="store_true",
+                    help="end-to-end leg: prompt lengths uniform in [P/2, 3P/2] so sequences reach "
+                         "their budget on different steps")
+    ap.add_argument("--separate-select-stages", action="store_true",
+                    help="run pooling, the mask epilogue and top-k as three launches (timed under "
+                         "the reference's stage names) instead of the one-launch selection")
+    ap.add_argument("--place-tries", type=int, default=16,
+                    help="most pool-sized allocations made side by side before any data is written "
+                         "(allocation stops as soon as a pair is fast or 160 GB are held); a timed "
+                         "compaction on pairs of them picks the K pool and the V pool (the "
+                         "in-place compaction is ~15 %% faster when the two lie in different regions "
+                         "of device memory); every probe figure is reported in 'placement' and the "
+                         "first-two-allocations figure in 'roofline'; 1 = take the first two "
+                         "allocations")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample", type=int, default=64)
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (read 1 GiB, write 1 GiB) so that a "
+                         "rocprofv3 --pmc run of this command has a kernel of known traffic to "
+                         "scale FETCH_SIZE / WRITE_SIZE by")
+    ap.add_argument("--traffic", type=float, default=None,
+                    help="HBM bytes per compaction launch measured with rocprofv3 --pmc "
+                         "(reported as roofline.traffic)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures the single-GPU hot path only; run with --gpus 1 "
+              "(every (sequence, kv head, layer) is independent, so more GPUs shard sequences "
+              "with no exchange step).", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from zipage_amd import _lib
+
+    _lib.load()  # fail loudly if the HIP library is missing
+    torch.cuda.set_device(0)
+    if args.config == 5:
+        e2e = end_to_end(args.requests, args.prompt, args.out_tokens, not args.sync_compress,
+                         args.ragged_prompts, args.script_switches)
+        print(json.dumps({
+            "metric": "decode tokens/sec", "value": e2e["decode_tok_per_s"], "unit": "tokens/s",
+            "n_gpus": 1, "steps": e2e["decode_steps"], "warmup": 0,
+            "ms_per_step": e2e["ms_per_decode_step"], "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": e2e["workload"]}, "roofline": e2e["decode_attention"],
+            "cpu_baseline": None, "end_to_end": e2e}))
+        return
+
     if args.calibrate_copy:
         src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
         dst = torch.empty_like(src)
@@ -273,65 +372,22 @@ def main():
             torch.mul(src, 1.0, out=dst)  # one streaming kernel: reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
         del src, dst
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    # timed region: only the roofline kernel carries events (each event pair costs the stream a
-    # few microseconds, 8 % of a step when every stage has one)
-    kv_timer = StageTimer(True, only=("compress_kv",))
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(kv_timer)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    # the per-stage breakdown comes from a second, untimed pass with events around every stage
-    timer = StageTimer(True)
-    for _ in range(args.steps):
-        step(timer)
-    torch.cuda.synchronize()
-
-    stage_s = timer.seconds()
-    ms_per_step = elapsed / args.steps * 1e3
-    seqs_per_s = wl.B / (elapsed / args.steps)
-    alg = algorithmic_bytes(wl, cfg)  # one layer
-    kv_s = kv_timer.seconds()["compress_kv"] / (args.steps * layers)
-    achieved = alg["compress_kv"] / kv_s / 1e9
-    stages_ms = {k: round(v / (args.steps * layers) * 1e3, 4) for k, v in stage_s.items()}
-    gpu_ms = sum(stage_s.values()) / (args.steps * layers) * 1e3  # per layer
-    out = {
-        "metric": "sequences compressed/sec",
-        "value": round(seqs_per_s, 1),
-        "unit": "sequences/s (one layer)" if layers == 1 else f"sequences/s ({layers} layers)",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if args.config == 3 else "bf16", "data": "synthetic",
-        "config": {"workload": desc, "batch": wl.B, "layers": layers},
-        "roofline": {"bound": "hbm", "kernel": "compact_kernel (compress_kv)",
-                     "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": args.traffic if args.traffic is not None
-                     else (COMPACT_TRAFFIC_PER_SEQ_LAYER * wl.B if wl.k.element_size() == 2
-                           else None),   # the counter runs were made on the bf16 workloads
-                     "algorithmic_bytes": alg["compress_kv"],
-                     "avg_launch_us": round(kv_s * 1e6, 2)},
-        "pipeline": {"algorithmic_bytes": alg["pipeline"],
-                     "gpu_ms_sum_of_stages_per_layer": round(gpu_ms, 4),
-                     "hbm_frac_of_stage_time": round(alg["pipeline"] / (gpu_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                     "stages_ms": stages_ms},
-    }
-    if wl.placement is not None:
-        out["placement"] = wl.placement
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(wl, cfg, min(args.cpu_sample, 16) if args.config == 3
-                                           else args.cpu_sample)
-    if not args.no_e2e and args.config == 2 and args.batch is None and sw == "pooling":
-        del wl
         torch.cuda.empty_cache()
-        out["end_to_end"] = end_to_end(args.requests, args.prompt, args.out_tokens,
-                                       not args.sync_compress, args.ragged_prompts,
-                                       args.script_switches)
+
+    run = run_pipeline(args.config, args, args.pipeline_switches, args.batch)
+    out = {"metric": "sequences compressed/sec", "value": run.pop("value"), "unit": run.pop("unit"),
+           "n_gpus": 1, "steps": run.pop("steps"), "warmup": run.pop("warmup"),
+           "ms_per_step": run.pop("ms_per_step"), "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": run.pop("dtype"), "data": "synthetic"}
+    out.update(run)
+    headline = args.config == 4 and args.batch is None
+    if headline and not args.no_extra_legs:
+        # the smaller single-layer workload of BASELINE configs[1], more steps (a step is 0.4 ms)
+        out["configs1_b64"] = run_pipeline(2, args, steps=max(args.steps, 100), warmup=10)
+        if not args.no_e2e:
+            out["end_to_end"] = end_to_end(args.requests, args.prompt, args.out_tokens,
+                                           not args.sync_compress, args.ragged_prompts,
+                                           args.script_switches)
     print(json.dumps(out))
 
 

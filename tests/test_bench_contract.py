@@ -19,12 +19,13 @@ def test_help_lists_the_contract_flags():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--help"],
                        capture_output=True, text=True, timeout=60)
     assert r.returncode == 0
-    for flag in ("--gpus", "--steps", "--warmup", "--config", "--no-e2e", "--pipeline-switches"):
+    for flag in ("--gpus", "--steps", "--warmup", "--config", "--no-e2e", "--no-extra-legs",
+                 "--pipeline-switches"):
         assert flag in r.stdout
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("extra", [["--config", "2"], ["--config", "3"],
+@pytest.mark.parametrize("extra", [["--config", "4"], ["--config", "2"], ["--config", "3"],
                                    ["--config", "2", "--pipeline-switches", "scripts"]])
 def test_bench_line_on_a_small_batch(extra):
     """One JSON line with the contract's keys, on a batch small enough for a test."""
@@ -46,4 +47,9 @@ def test_bench_line_on_a_small_batch(extra):
     assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
     assert out["cpu_baseline"]["kind"] == "port" and out["cpu_baseline"]["value"] > 0
     assert out["placement"]["slabs"] == 2
+    first = roof["first_two_allocations"]
+    assert abs(first["frac"] - first["achieved"] / roof["peak"]) < 1e-3
+    assert "traffic" in roof and "traffic_source" in roof
+    if extra == ["--config", "4"]:
+        assert out["config"]["layers"] == 36 and "36 layers" in out["unit"]
     assert "workload" in out["config"] and "model" not in out["config"]
