@@ -76,12 +76,18 @@ int64_t zp_attention_score_workspace(int32_t L, int32_t B, int32_t NB, int32_t B
  * zipage/kernel/global_score.py:77-120 (kernel :8-74).
  * scores (L, B, Hkv, NB, BS) contiguous, updated in place; score_cache
  * (L, num_pages, BS, Hkv) with the given layer/page strides, slot stride Hkv, head
- * stride 1; compressed: B bytes (bool). */
+ * stride 1; compressed: B bytes (bool).
+ * write_cache != 0 is the reference: every sequence's result is also stored to its pages of
+ * the score cache (global_score.py:73-74).  When several sequences of the batch share a page
+ * (prefix cache) those stores race, and compress_score would read back whichever landed last;
+ * with write_cache == 0 the cache is only read, and zp_compress_score(scores_src = scores)
+ * takes the carried values from `scores` instead, which is deterministic and equal to the
+ * reference whenever no page is shared. */
 int zp_global_score(void* scores, void* score_cache, const int32_t* block_table,
                     const uint8_t* compressed, int32_t L, int32_t B, int32_t NB,
                     int32_t BS, int32_t Hkv, int32_t num_pages, int64_t c_stride_layer,
                     int64_t c_stride_page, float decay_factor, int32_t activate_method,
-                    int32_t dtype, void* stream);
+                    int32_t write_cache, int32_t dtype, void* stream);
 
 /* Sequence-axis pooling done inline by the runner:
  * zipage/engine/model_runner.py:499-530  (F.max_pool1d, stride 1, pad kernel//2, then
@@ -177,8 +183,12 @@ int zp_compress_kv(void* key, void* value, const uint8_t* flag, const int32_t* b
                    int32_t dtype, void* stream);
 
 /* compress_score(score_cache, flag, block_table, target_block_table)
- * zipage/kernel/compress_score.py:66-99 (kernel :8-63). */
-int zp_compress_score(void* score_cache, const uint8_t* flag, const int32_t* block_table,
+ * zipage/kernel/compress_score.py:66-99 (kernel :8-63).
+ * scores_src NULL: the reference (each kept token's value is read from its source page of the
+ * score cache).  scores_src = the (L, B, Hkv, NB, BS) scores zp_global_score left: the value
+ * of a kept token is read from there (see zp_global_score, write_cache). */
+int zp_compress_score(void* score_cache, const void* scores_src, const uint8_t* flag,
+                      const int32_t* block_table,
                       const int32_t* target_block_table, int32_t L, int32_t B, int32_t NB,
                       int32_t BS, int32_t Hkv, int32_t num_pages, int32_t target_width,
                       int64_t c_stride_layer, int64_t c_stride_page, int64_t c_stride_slot,

@@ -139,12 +139,15 @@ def attention_score(k_cache, query_cache, seq_idx, block_table, softmax_scale=No
 
 # -------------------------------------------------------------------- a3 global score
 def global_score(reduced_scores, score_cache, block_table, compressed, decay_factor=0.9,
-                 activate_method="max"):
+                 activate_method="max", write_cache=True):
     """Carry scores over from the previous compression (global_score.py:8-74,77-120).
     For a non-pad page of a sequence that is ``compressed`` and is not its last page:
     ``out = max(new, old*decay)`` or ``new + old*decay`` in fp32, cast to the scores'
     dtype (:60-70); otherwise ``out = new``.  ``out`` goes to the scores in place and to
-    ``score_cache[l, page, slot, head]`` (:73-74)."""
+    ``score_cache[l, page, slot, head]`` (:73-74).  The loop visits sequences in order, so a
+    page several sequences share ends up with the LAST sequence's scores (on a GPU the
+    reference's stores race).  ``write_cache=False`` is this build's race-free mode: the cache
+    is only read (see :func:`compress_score`, ``scores_src``)."""
     assert 0 <= decay_factor <= 1
     assert activate_method in ("max", "sum")
     decay = float(torch.tensor(decay_factor, dtype=torch.float32))
@@ -165,7 +168,8 @@ def global_score(reduced_scores, score_cache, block_table, compressed, decay_fac
             else:
                 out = new.clone()
             reduced_scores[:, b, :, j, :] = out
-            score_cache[:, pid] = out.permute(0, 2, 1).to(score_cache.dtype)
+            if write_cache:
+                score_cache[:, pid] = out.permute(0, 2, 1).to(score_cache.dtype)
     return reduced_scores
 
 
@@ -447,9 +451,13 @@ def compress_kv(key, value, flag, block_table, target_block_table) -> None:
                 value[l, dp, ds, h] = vv
 
 
-def compress_score(score_cache, flag, block_table, target_block_table):
+def compress_score(score_cache, flag, block_table, target_block_table, scores_src=None):
     """Same walk moving one ``score_cache[l, page, slot, head]`` scalar per kept token
-    (compress_score.py:8-63,66-99)."""
+    (compress_score.py:8-63,66-99).  With ``scores_src`` ``(L,B,Hkv,NB,BS)`` (this build's
+    race-free mode, no counterpart in the reference) the scalar of a kept token is taken from
+    there: it is what ``global_score`` would have stored for THIS sequence, so the result
+    equals the reference's whenever no source page is shared with another sequence of the
+    batch, and does not depend on the order of the sequences when one is."""
     L, _, BS, Hkv = score_cache.shape
     _, B, _, NB, _ = flag.shape
     for l in range(L):
@@ -458,6 +466,13 @@ def compress_score(score_cache, flag, block_table, target_block_table):
                 sp, ss, dp, ds = _compaction_plan(flag[l, b, h], block_table[b],
                                                   target_block_table[b], BS)
                 if not sp:
+                    continue
+                if scores_src is not None:
+                    # logical (page index, slot) of every kept token, in the walk's order
+                    kept = [(j, s) for j, code in enumerate(block_table[b].tolist()) if code != -1
+                            for s in torch.nonzero(flag[l, b, h, j]).flatten().tolist()]
+                    vals = torch.stack([scores_src[l, b, h, j, s] for j, s in kept])
+                    score_cache[l, torch.tensor(dp), torch.tensor(ds), h] = vals.to(score_cache.dtype)
                     continue
                 vals = score_cache[l, torch.tensor(sp), torch.tensor(ss), h].clone()
                 score_cache[l, torch.tensor(dp), torch.tensor(ds), h] = vals
@@ -473,12 +488,15 @@ def compress_pipeline(k_cache, v_cache, query_cache, score_cache, query_ids, blo
                       pooling_mode="max", use_redudancy=False, lightning_redudancy=False,
                       redudancy_lambda=0.2, redudancy_temperature=0.4,
                       redudancy_threshold=0.5, use_attention_sink=False, sink_len=4,
-                      rounding="reference", return_intermediates=False):
+                      rounding="reference", return_intermediates=False,
+                      deterministic_carry=False):
     """One layer chunk of ``ModelRunner.compress`` (model_runner.py:466-622), same stage
     order: attention_score -> [max-norm] global_score -> pooling -> redundancy + combine
     -> sink -> window_mask -> pad mask -> top-k (k = BS*budget) -> compress_kv ->
     compress_score.  Mutates ``k_cache``, ``v_cache`` and ``score_cache`` in place and
-    returns the keep flag (and the final scores when asked)."""
+    returns the keep flag (and the final scores when asked).  ``deterministic_carry`` is this
+    build's race-free handling of the score cache: ``global_score`` only reads it and the
+    carried scores of the survivors are compacted from the scores it returned."""
     BS = k_cache.shape[2]
     scores = attention_score(k_cache, query_cache, query_ids, block_table, softmax_scale,
                              reduced, rounding=rounding)
@@ -486,7 +504,8 @@ def compress_pipeline(k_cache, v_cache, query_cache, score_cache, query_ids, blo
         if max_norm:
             scores = max_normalise(scores)
         scores = global_score(scores, score_cache, block_table, compressed, decay_factor,
-                              activate_method)
+                              activate_method, write_cache=not deterministic_carry)
+        carried = scores.clone() if deterministic_carry else None
     if enable_pooling:
         scores = pool_scores(scores, compressed, pooling_size, continues_pooling,
                              pooling_mode)
@@ -506,7 +525,7 @@ def compress_pipeline(k_cache, v_cache, query_cache, score_cache, query_ids, blo
     flag = flag.view(L, B, Hkv, NB, BS)
     compress_kv(k_cache, v_cache, flag, block_table, target_block_table)
     if use_global_score:
-        compress_score(score_cache, flag, block_table, target_block_table)
+        compress_score(score_cache, flag, block_table, target_block_table, scores_src=carried)
     if return_intermediates:
         return flag, scores
     return flag

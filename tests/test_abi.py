@@ -37,7 +37,7 @@ def test_library_exports_every_declared_symbol():
 def test_version_and_error_string():
     from zipage_amd import _lib
     lib = _lib.load()
-    assert lib.zp_abi_version() >= 1
+    assert lib.zp_abi_version() >= 2
     assert isinstance(lib.zp_last_error(), bytes)
 
 
@@ -47,7 +47,7 @@ def test_argument_validation_needs_no_gpu():
     lib = _lib.load()
     rc = lib.zp_topk_mask(None, None, 4, 16, 17, 0, None)
     assert rc == 1 and b"k=17" in lib.zp_last_error()
-    rc = lib.zp_global_score(1, 1, 1, 1, 1, 1, 1, 256, 8, 4, 0, 0, 1.5, 0, 0, None)
+    rc = lib.zp_global_score(1, 1, 1, 1, 1, 1, 1, 256, 8, 4, 0, 0, 1.5, 0, 1, 0, None)
     assert rc == 1 and b"decay_factor" in lib.zp_last_error()
 
 

@@ -20,6 +20,10 @@ _spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(HER
 mf = importlib.util.module_from_spec(_spec)
 _spec.loader.exec_module(mf)
 
+# at most twice what the committed cases show on MI355X (printed by every run: pytest -s)
+SCORE_OUTLIERS_16BIT = 5e-4   # observed: 0
+FLAG_MISMATCH_16BIT = 2e-3    # observed: 0
+
 with open(os.path.join(HERE, "golden", "compress_cases.json")) as f:
     FIXTURES = json.load(f)
 
@@ -72,7 +76,8 @@ def test_hip_pipeline_reproduces_the_committed_vectors(dev, fx):
     fin = torch.isfinite(ws)
     rel = 1e-3 if dtype == torch.float32 else 2.0 ** -6
     bad = ((gs[fin] - ws[fin]).abs() > rel * ws[fin].abs() + 1e-8).float().mean().item()
-    assert bad <= (0.0 if dtype == torch.float32 else 2e-3), f"{bad} of scores off"
+    print(f"  scores beyond rel {rel:.2e} of the stored vectors: {bad:.2e}")
+    assert bad <= (0.0 if dtype == torch.float32 else SCORE_OUTLIERS_16BIT), f"{bad} of scores off"
     assert (gflag.flatten(3).sum(-1) == fx["kept_per_row"]).all()
     diff = gflag != flag
     if diff.any():   # only where the stored scores are near-tied with the k-th one
@@ -81,7 +86,8 @@ def test_hip_pipeline_reproduces_the_committed_vectors(dev, fx):
         kth = flat.topk(fx["kept_per_row"], dim=-1).values[..., -1:].expand_as(flat).reshape_as(ws)
         gap = (ws - kth).abs()[diff]
         assert (gap <= 4 * rel * kth[diff].abs() + 1e-8).all()
-        assert diff.float().mean().item() <= 2e-2
+        print(f"  keep flags differing from the stored flags: {diff.float().mean().item():.2e}")
+        assert diff.float().mean().item() <= FLAG_MISMATCH_16BIT
     else:
         tgt = inp["target"][:, :c["budget"]].flatten().long()
         got = mf.sha(k.cpu()[:, tgt], v.cpu()[:, tgt], None if sc is None else sc.cpu()[:, tgt])

@@ -18,6 +18,8 @@ from oracle import zipage_oracle as O
 pytestmark = pytest.mark.gpu
 
 BS, BUDGET = 256, 8
+# at most twice what the sampled sequences show on MI355X (printed by every run: pytest -s)
+SCORE_OUTLIERS_16BIT = 5e-4   # observed: 0
 
 
 def _run_pipeline(wl, cfg):
@@ -91,7 +93,8 @@ def _oracle_sample(wl, sub, cfg_kwargs, seq_ids, scores_gpu, dtype):
     fin = torch.isfinite(w)
     rel = 1e-3 if dtype == torch.float32 else 2.0 ** -6
     bad = ((g[fin] - w[fin]).abs() > rel * w[fin].abs() + 1e-9).float().mean().item()
-    assert bad <= (0.0 if dtype == torch.float32 else 2e-3), f"{bad} of sampled scores off"
+    print(f"  sampled scores beyond rel {rel:.2e}: {bad:.2e}")
+    assert bad <= (0.0 if dtype == torch.float32 else SCORE_OUTLIERS_16BIT), f"{bad} of sampled scores off"
 
 
 def test_config2_64_ragged_sequences(dev):
@@ -157,22 +160,28 @@ def test_config1_single_sequence_fp32_full_oracle(dev):
     assert ((g[fin] - w[fin]).abs() <= 1e-3 * w[fin].abs() + 1e-10).all()
     assert torch.equal(flag.cpu(), O.topk_mask(scores.cpu().view(1, 1, 8, -1), 2048).view_as(flag))
     mism = (flag.cpu() != oflag).float().mean().item()
-    assert mism <= 1e-3
+    print(f"  keep flags differing from the oracle's end-to-end flags: {mism:.2e}")
+    assert mism <= 1e-4    # observed: 0
     if mism == 0:
         pages = torch.tensor(sub["pages"], device=wl.k.device)
         assert torch.equal(wl.k[:, pages].cpu(), sub["k"]) and torch.equal(wl.v[:, pages].cpu(), sub["v"])
 
 
-def test_config3_global_score_and_redundancy_128_sequences(dev):
-    """BASELINE configs[2]: configs[0] shape and dtype, 128 sequences, carried global score
-    (decay 0.9) and lightning redundancy; properties on the batch, oracle on two sequences."""
+@pytest.mark.parametrize("variant", ["lightning", "raw"])
+def test_config3_global_score_and_redundancy_128_sequences(dev, variant):
+    """BASELINE configs[2] with exactly the switches `bench.py --config 3` times: configs[0]
+    shape and dtype (fp32), 128 sequences, carried global score ADDED with decay 0.9
+    (activate_method "sum"), avg-pool 7 on every sequence (continues_pooling), score minus 0.5 x
+    redundancy (lambda 2/3), lightning or all-pairs redundancy; properties on the whole batch,
+    the oracle's full pipeline on two of the sequences."""
     from zipage_amd.compress import CompressConfig
     from zipage_amd.workload import QWEN3_0_6B, cpu_subset, ragged_batch
-    wl = ragged_batch(128, L=1, pool_pages=2000, budget=BUDGET, W=32, seed=2, lengths=(2304, 2304),
+    wl = ragged_batch(128, L=1, pool_pages=2048, budget=BUDGET, W=32, seed=0, lengths=(2304, 2304),
                       dtype=torch.float32, shape=QWEN3_0_6B, with_score_cache=True, compressed=True)
     kb, vb = _save_touched(wl)
-    kw = dict(use_global_score=True, decay_factor=0.9, use_redudancy=True, lightning_redudancy=True,
-              redudancy_lambda=0.5, enable_pooling=True, pooling_size=7, continues_pooling=True)
+    kw = dict(use_global_score=True, decay_factor=0.9, activate_method="sum", use_redudancy=True,
+              lightning_redudancy=variant == "lightning", redudancy_lambda=2.0 / 3.0,
+              enable_pooling=True, pooling_size=7, continues_pooling=True, pooling_mode="avg")
     ids = [5, 100]
     sub = cpu_subset(wl, ids)
     oflag, oscores = O.compress_pipeline(
@@ -184,4 +193,8 @@ def test_config3_global_score_and_redundancy_128_sequences(dev):
     g, w = scores[:, ids].float().cpu(), oscores.float()
     fin = torch.isfinite(w)
     assert torch.equal(torch.isinf(g), torch.isinf(w))
+    err = ((g[fin] - w[fin]).abs() / (w[fin].abs() + 1e-8)).max().item()
+    mism = (flag[:, ids].cpu() != oflag).float().mean().item()
+    print(f"  worst relative score error {err:.2e}; keep flags differing from the oracle's: {mism:.2e}")
     assert ((g[fin] - w[fin]).abs() <= 1e-3 * w[fin].abs() + 1e-8).all()
+    assert mism <= 1e-3

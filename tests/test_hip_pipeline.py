@@ -18,9 +18,16 @@ from tests import cases
 
 pytestmark = pytest.mark.gpu
 
+# Bounds on what may differ from the oracle, at most twice what the cases below show on MI355X
+# (printed by every run: pytest -s).  16-bit: a logit whose fp32 sum falls on the other side of a
+# rounding boundary moves its score by a few units in the last place; fp32: nothing may differ.
+SCORE_OUTLIERS = {torch.float32: 0.0, torch.bfloat16: 3e-3}    # observed: 0 and 1.5e-3
+FLAG_MISMATCH = {torch.float32: 0.0, torch.bfloat16: 6e-3}     # observed: 0 and 2.7e-3
+
 
 def _run(dev, dtype, cfg_kwargs, seed=61, L=2, B=4, Hkv=2, Hq=8, W=32, budget=2,
-         nb_choices=(3, 4), num_pages=40, compressed=(False, True, False, True)):
+         nb_choices=(3, 4), num_pages=40, compressed=(False, True, False, True),
+         deterministic_carry=True):
     from zipage_amd.compress import CompressConfig, compress_layers
     tables, enc, target = cases.random_tables(seed, B, num_pages, list(nb_choices), budget)
     k, v, q, sc = cases.make_caches(seed, L, num_pages, 256, Hkv, Hq, 128, W, B + 1, dtype,
@@ -35,11 +42,12 @@ def _run(dev, dtype, cfg_kwargs, seed=61, L=2, B=4, Hkv=2, Hq=8, W=32, budget=2,
     ok, ov, osc = k.clone(), v.clone(), sc.clone()
     oflag, oscores = O.compress_pipeline(
         ok, ov, q, osc, qid, enc, comp, target, budget_blocks=budget, query_cache_len=W,
-        return_intermediates=True, **cfg_kwargs)
+        return_intermediates=True, deterministic_carry=deterministic_carry, **cfg_kwargs)
 
     gk, gv, gsc = k.clone().to(dev), v.clone().to(dev), sc.clone().to(dev)
     gflag, gscores = compress_layers(gk, gv, q.to(dev), gsc, qid.to(dev), enc.to(dev),
-                                     comp.to(dev), target.to(dev), cfg, return_intermediates=True)
+                                     comp.to(dev), target.to(dev), cfg, return_intermediates=True,
+                                     deterministic_carry=deterministic_carry)
     gflag, gscores = gflag.cpu(), gscores.cpu()
     BS = 256
     NB = enc.shape[1]
@@ -53,7 +61,8 @@ def _run(dev, dtype, cfg_kwargs, seed=61, L=2, B=4, Hkv=2, Hq=8, W=32, budget=2,
     err = (gs[fin] - os_[fin]).abs()
     tol = rel * os_[fin].abs() + 1e-9
     frac_bad = (err > tol).float().mean().item()
-    assert frac_bad <= (0.0 if dtype == torch.float32 else 2e-3), f"{frac_bad} of scores off"
+    print(f"  scores beyond rel {rel:.2e}: {frac_bad:.2e} (bound {SCORE_OUTLIERS[dtype]:.1e})")
+    assert frac_bad <= SCORE_OUTLIERS[dtype], f"{frac_bad} of scores off"
 
     # (ii) selector on the GPU's own scores
     want_flag = O.topk_mask(gscores.view(L, B, Hkv, NB * BS), kk).view_as(gflag)
@@ -68,26 +77,31 @@ def _run(dev, dtype, cfg_kwargs, seed=61, L=2, B=4, Hkv=2, Hq=8, W=32, budget=2,
         gap = (os_ - kth).abs()[diff]
         assert (gap <= 4 * rel * kth[diff].abs() + 1e-9).all(), "flag differs away from the k-th score"
     mism = diff.float().mean().item()
-    assert mism <= (1e-4 if dtype == torch.float32 else 2e-2)
+    print(f"  keep flags differing from the oracle's end-to-end flags: {mism:.2e} "
+          f"(bound {FLAG_MISMATCH[dtype]:.1e})")
+    assert mism <= FLAG_MISMATCH[dtype]
 
     # (iv) compaction driven by the GPU flag
     ck, cv, csc = k.clone(), v.clone(), sc.clone()
     if cfg.use_global_score:
-        # the score cache the compaction reads is the one global_score wrote
+        # reference mode: the score cache the compaction reads is the one global_score wrote;
+        # deterministic mode: the cache is only read and the compaction takes the scores
         s2 = O.attention_score(k, q, qid, enc, None, cfg.reduced)
         if cfg.max_norm:
             s2 = O.max_normalise(s2)
-        O.global_score(s2, csc, enc, comp, cfg.decay_factor, cfg.activate_method)
+        O.global_score(s2, csc, enc, comp, cfg.decay_factor, cfg.activate_method,
+                       write_cache=not deterministic_carry)
     O.compress_kv(ck, cv, gflag, enc, target)
     assert torch.equal(gk.cpu().view(torch.uint8), ck.view(torch.uint8))
     assert torch.equal(gv.cpu().view(torch.uint8), cv.view(torch.uint8))
     if cfg.use_global_score:
         # carried scores: same walk; values agree to the score tolerance
-        O.compress_score(csc, gflag, enc, target)
+        O.compress_score(csc, gflag, enc, target, scores_src=s2 if deterministic_carry else None)
         touched = sorted(cases.touched_pages(enc))
         a, b_ = gsc.cpu().float()[:, touched], csc.float()[:, touched]
         bad = ((a - b_).abs() > rel * b_.abs() + 1e-9).float().mean().item()
-        assert bad <= (0.0 if dtype == torch.float32 else 2e-3), f"{bad} of carried scores off"
+        print(f"  carried scores beyond rel {rel:.2e}: {bad:.2e}")
+        assert bad <= SCORE_OUTLIERS[dtype], f"{bad} of carried scores off"
     return dict(mismatch=mism)
 
 
@@ -99,11 +113,84 @@ def test_pipeline_score_pool_topk_compact(dev, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("lightning", [True, False])
-def test_pipeline_global_and_redundancy(dev, dtype, lightning):
-    """BASELINE config 3 pipeline: global score (decay 0.9), redundancy, combine, pooling."""
+@pytest.mark.parametrize("deterministic_carry", [True, False])
+def test_pipeline_global_and_redundancy(dev, dtype, lightning, deterministic_carry):
+    """BASELINE config 3 pipeline: global score (decay 0.9), redundancy, combine, pooling; with
+    the carried scores compacted from the scores (default) and read back from the score cache
+    as the reference does."""
     _run(dev, dtype, dict(use_global_score=True, decay_factor=0.9, enable_pooling=True,
                           pooling_size=7, use_redudancy=True, lightning_redudancy=lightning,
-                          redudancy_lambda=0.5))
+                          redudancy_lambda=0.5), deterministic_carry=deterministic_carry)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_pipeline_bench_config3_switches(dev, dtype):
+    """The switch set `bench.py --config 3` times: carried score added with decay 0.9, avg-pool 7
+    on every sequence, score minus 0.5 x redundancy (lambda 2/3)."""
+    for lightning in (True, False):
+        _run(dev, dtype, dict(use_global_score=True, decay_factor=0.9, activate_method="sum",
+                              enable_pooling=True, continues_pooling=True, pooling_size=7,
+                              pooling_mode="avg", use_redudancy=True, lightning_redudancy=lightning,
+                              redudancy_lambda=2.0 / 3.0))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_shared_prefix_with_global_score_is_deterministic(dev, dtype):
+    """Sequences that share prefix pages (first compression, copy-on-write targets) next to an
+    already-compressed one, global score on.  The reference stores every sequence's scores into
+    the shared page of the score cache and reads them back for the compaction
+    (zipage/kernel/global_score.py:73-74, zipage/kernel/compress_score.py:50-53), so its carried
+    scores depend on which store landed last.  Here each sequence carries its OWN scores: equal
+    to the oracle's race-free mode, identical on every run, different from the oracle's
+    sequential reference mode exactly on tokens kept from shared pages, and the shared pages of
+    K, V and the score cache are never written."""
+    from zipage_amd.compress import CompressConfig, compress_layers
+    L, Hkv, Hq, W, budget, BS, num_pages = 2, 2, 8, 16, 2, 256, 40
+    # two groups of two sequences sharing their first page, then one compressed sequence
+    tables = [[0, 2, 3, 4], [0, 5, 6], [1, 7, 8, 9], [1, 10, 11, 12], [13, 14, 15]]
+    targets = [[20, 2, 3], [21, 5, 6], [22, 7, 8], [23, 10, 11], [13, 14, 15]]
+    comp = torch.tensor([False, False, False, False, True])
+    B = len(tables)
+    enc = O.encode_block_table(tables)
+    target = torch.tensor(targets, dtype=torch.int32)
+    k, v, q, sc = cases.make_caches(7, L, num_pages, BS, Hkv, Hq, 128, W, B, dtype,
+                                    touched=cases.touched_pages(enc), with_score_cache=True)
+    qid = torch.arange(B, dtype=torch.int32)
+    kw = dict(use_global_score=True, decay_factor=0.8, enable_pooling=True, pooling_size=5)
+    cfg = CompressConfig(budget_blocks=budget, query_cache_len=W, **kw)
+
+    def run_gpu():
+        gk, gv, gsc = k.clone().to(dev), v.clone().to(dev), sc.clone().to(dev)
+        flag = compress_layers(gk, gv, q.to(dev), gsc, qid.to(dev), enc.to(dev), comp.to(dev),
+                               target.to(dev), cfg)
+        return flag.cpu(), gk.cpu(), gv.cpu(), gsc.cpu()
+
+    f1, k1, v1, c1 = run_gpu()
+    f2, k2, v2, c2 = run_gpu()
+    for a, b_ in ((f1, f2), (k1, k2), (v1, v2), (c1, c2)):
+        assert torch.equal(a.view(torch.uint8), b_.view(torch.uint8)), "two runs differ"
+    for p in (0, 1):
+        assert torch.equal(k1[:, p], k[:, p]) and torch.equal(v1[:, p], v[:, p])
+        assert torch.equal(c1[:, p], sc[:, p]), "a shared page of the score cache was written"
+
+    # the oracle, race-free mode, driven by the GPU's flags (selection parity is covered above)
+    s2 = O.attention_score(k, q, qid, enc)
+    want = sc.clone()
+    O.global_score(s2, want, enc, comp, 0.8, "max", write_cache=False)
+    O.compress_score(want, f1, enc, target, scores_src=s2)
+    rel = 1e-3 if dtype == torch.float32 else 2.0 ** -6
+    bad = ((c1.float() - want.float()).abs() > rel * want.float().abs() + 1e-9).float().mean().item()
+    print(f"  carried scores beyond rel {rel:.2e}: {bad:.2e}")
+    assert bad <= SCORE_OUTLIERS[dtype]
+    # and the sequential reference mode differs on the first sequence of each group only where
+    # tokens were kept from the shared page (whose cache the second sequence overwrote)
+    ref = sc.clone()
+    s3 = O.attention_score(k, q, qid, enc)
+    O.global_score(s3, ref, enc, comp, 0.8, "max")
+    O.compress_score(ref, f1, enc, target)
+    d = (ref.float() - want.float()).abs() > rel * want.float().abs() + 1e-9
+    assert d[:, [20, 22]].any(), "the case does not exercise the shared-page read-back"
+    assert not d[:, [21, 23, 13, 14]].any()
 
 
 def test_pipeline_shipping_defaults(dev):

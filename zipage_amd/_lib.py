@@ -27,7 +27,7 @@ SIGNATURES = {
     "zp_attention_score": [ptr, ptr, ptr, ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32, i32,
                            i32, i32, i64, i64, i64, i64, f32, i32, i32, ptr, i64, ptr],
     "zp_global_score": [ptr, ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i64, i64, f32, i32, i32,
-                        ptr],
+                        i32, ptr],
     "zp_pool_scores": [ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32, i32, ptr],
     "zp_key_norm": [ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32, i64, i64, f32, i32, ptr],
     "zp_redundancy_lightning": [ptr, ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32, i64, i64,
@@ -41,7 +41,7 @@ SIGNATURES = {
                        f64, i32, i32, i32, i32, i32, ptr],
     "zp_compress_kv": [ptr, ptr, ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32, i32,
                        i64, i64, i64, i64, i64, i64, i64, i64, i32, ptr],
-    "zp_compress_score": [ptr, ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32, i64, i64, i64,
+    "zp_compress_score": [ptr, ptr, ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32, i64, i64, i64,
                           i64, i32, ptr],
     "zp_store_kvcache": [ptr, ptr, ptr, ptr, ptr, i32, i32, i64, i64, i64, i32, ptr],
     "zp_paged_decode_attention": [ptr, ptr, ptr, ptr, ptr, ptr, i32, i32, i32, i32, i32, i32, i32,

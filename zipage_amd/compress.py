@@ -89,13 +89,22 @@ class StageTimer:
 
 def compress_layers(k_cache, v_cache, query_cache, score_cache, query_ids, block_tables,
                     compressed, target_block_tables, cfg: CompressConfig, timer=None,
-                    return_intermediates=False, fused_select=True):
+                    return_intermediates=False, fused_select=True, deterministic_carry=True):
     """Score, select and compact one chunk of layers in place.
 
     k_cache/v_cache: (L, num_pages, BS, Hkv, D); query_cache: (L, max_seqs, W, Hq, D);
     score_cache: (L, num_pages, BS, Hkv) or None; query_ids: (B,) int32; block_tables:
     (B, NB) int32 encoded as in model_runner.py:437-463; compressed: (B,) bool;
     target_block_tables: (B, budget+1) int32.  Returns the keep flag (L, B, Hkv, NB, BS).
+
+    ``deterministic_carry`` (default): the reference's global_score stores every sequence's
+    scores into its pages of the score cache (global_score.py:73-74) and compress_score reads
+    them back (compress_score.py:50-53); when sequences of the batch share prefix pages those
+    stores race and the carried scores depend on the order the GPU ran them in.  Here the
+    score cache is only read by global_score and the survivors' carried scores are compacted
+    straight from the scores it returned: the same values as the reference whenever no page is
+    shared, independent of scheduling when one is, and no shared (read-only) page is written.
+    ``False`` runs the reference's two stores.
     """
     t = timer or StageTimer(False)
     BS = k_cache.shape[2]
@@ -110,8 +119,9 @@ def compress_layers(k_cache, v_cache, query_cache, score_cache, query_ids, block
         if cfg.max_norm:
             score_epilogue(scores, block_tables, max_norm_scores=True)
         scores = global_score(scores, score_cache, block_tables, compressed, cfg.decay_factor,
-                              cfg.activate_method)
+                              cfg.activate_method, write_cache=not deterministic_carry)
         t.stop(ev)
+    carried = scores if (cfg.use_global_score and deterministic_carry) else None
 
     red = None
     if cfg.use_redudancy:
@@ -136,6 +146,8 @@ def compress_layers(k_cache, v_cache, query_cache, score_cache, query_ids, block
         flag, scores = out if return_intermediates else (out, scores)
         t.stop(ev)
     else:
+        if carried is not None and not cfg.enable_pooling:
+            carried = scores.clone()   # the mask epilogue below works in place on `scores`
         if cfg.enable_pooling:
             ev = t.start("pooling")
             scores = pool_scores(scores, compressed, cfg.pooling_size, cfg.continues_pooling,
@@ -162,7 +174,7 @@ def compress_layers(k_cache, v_cache, query_cache, score_cache, query_ids, block
 
     if cfg.use_global_score:
         ev = t.start("compress_global_score")
-        compress_score(score_cache, flag, block_tables, target_block_tables)
+        compress_score(score_cache, flag, block_tables, target_block_tables, scores_src=carried)
         t.stop(ev)
     if return_intermediates:
         return flag, scores

@@ -59,6 +59,9 @@ struct CompactArgs {
   int bs_shift;        // log2(BS) or -1
   int64_t a_sl, a_sp, a_ss, a_sh;  // byte strides: layer, page, slot, head
   int64_t b_sl, b_sp, b_ss, b_sh;
+  // score compaction only: when set, the value of logical token s of row (l, b, h) is read from
+  // rows[((l*B + b)*Hkv + h)*T + s] (elements of sizeof(P)) instead of from `a` through the table
+  const char* rows;
 };
 
 // Survivors are written once and not read again by this kernel: non-temporal stores keep them
@@ -132,7 +135,10 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
       const int s = list[i];
       const int j = page_of(s), slot = s - j * p.BS;
       const int64_t pid = tab[j];
-      ra[r] = ZP_NT_LOAD((const P*)(abase + pid * p.a_sp + slot * p.a_ss + piece * (int)sizeof(P)));
+      if (!HAS_B && p.rows)
+        ra[r] = *(const P*)(p.rows + ((int64_t)item * T + s) * (int)sizeof(P));
+      else
+        ra[r] = ZP_NT_LOAD((const P*)(abase + pid * p.a_sp + slot * p.a_ss + piece * (int)sizeof(P)));
       if (HAS_B)
         rb[r] = ZP_NT_LOAD((const P*)(bbase + pid * p.b_sp + slot * p.b_ss + piece * (int)sizeof(P)));
     }
@@ -229,7 +235,7 @@ extern "C" int zp_compress_kv(void* key, void* value, const uint8_t* flag,
   const int es = zp_dtype_bytes(dtype);
   CompactArgs a;
   a.a = (char*)key; a.b = (char*)value; a.flag = flag; a.table = block_table;
-  a.target = target_block_table;
+  a.target = target_block_table; a.rows = nullptr;
   a.B = B; a.NB = NB; a.BS = BS; a.Hkv = Hkv; a.num_pages = num_pages;
   a.target_width = target_width;
   a.a_sl = k_sl * es; a.a_sp = k_sp * es; a.a_ss = k_ss * es; a.a_sh = k_sh * es;
@@ -254,7 +260,7 @@ extern "C" int zp_compress_kv(void* key, void* value, const uint8_t* flag,
   }
 }
 
-extern "C" int zp_compress_score(void* score_cache, const uint8_t* flag,
+extern "C" int zp_compress_score(void* score_cache, const void* scores_src, const uint8_t* flag,
                                  const int32_t* block_table, const int32_t* target_block_table,
                                  int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
                                  int32_t num_pages, int32_t target_width, int64_t c_sl,
@@ -272,7 +278,7 @@ extern "C" int zp_compress_score(void* score_cache, const uint8_t* flag,
   const int es = zp_dtype_bytes(dtype);
   CompactArgs a;
   a.a = (char*)score_cache; a.b = nullptr; a.flag = flag; a.table = block_table;
-  a.target = target_block_table;
+  a.target = target_block_table; a.rows = (const char*)scores_src;
   a.B = B; a.NB = NB; a.BS = BS; a.Hkv = Hkv; a.num_pages = num_pages;
   a.target_width = target_width; a.lpv = 1;
   a.a_sl = c_sl * es; a.a_sp = c_sp * es; a.a_ss = c_ss * es; a.a_sh = c_sh * es;

@@ -960,7 +960,9 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
 #pragma unroll 1
     for (int j = g; j < p.BS; j += kPageThreads / PIECES) {
       const int c = l_col[j];
-      if (c < 0) continue;      // uniform over the 16 lanes of a key
+      // c == j: with a negative threshold the zeroed diagonal entry itself can be the claim; its
+      // value is 0, nothing to hand back
+      if (c < 0 || c == j) continue;      // uniform over the 16 lanes of a key
       const u32x4 kj = *(const u32x4*)(k_pl + j * ROWH + piece * 16);
       const u32x4 kc = *(const u32x4*)(k_pl + c * ROWH + piece * 16);
       float ej[8], ec[8];
@@ -1344,6 +1346,10 @@ __global__ __launch_bounds__(kThreads) void raw_claim_value_kernel(GramArgs p) {
     const int64_t oi = obase + (int64_t)jp * p.BS + slot;
     const int c = p.ws_col[oi];
     if (c < 0 || c >= Tn) continue;     // uniform over the 16 lanes of a key
+    if (c == jp * p.BS + slot) {        // negative threshold: the zeroed diagonal entry was claimed
+      if (piece == 0) p.ws_val[oi] = 0.f;
+      continue;
+    }
     const int cp = c / p.BS, cs = c - cp * p.BS;
     const int ccode = p.table[(int64_t)b * p.NB + cp];
     const int cpid = page_is_pad(ccode) ? -1 : page_id(ccode);

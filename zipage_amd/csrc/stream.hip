@@ -17,7 +17,7 @@ template <typename T>
 __global__ __launch_bounds__(kThreads) void global_score_kernel(
     void* __restrict__ scores, void* __restrict__ cache, const int32_t* __restrict__ table,
     const uint8_t* __restrict__ compressed, int B, int NB, int BS, int Hkv, int num_pages,
-    int64_t c_sl, int64_t c_sp, float decay, int method) {
+    int64_t c_sl, int64_t c_sp, float decay, int method, int write_cache) {
   const int j = blockIdx.x % NB;
   const int b = (blockIdx.x / NB) % B;
   const int l = blockIdx.x / (NB * B);
@@ -26,6 +26,7 @@ __global__ __launch_bounds__(kThreads) void global_score_kernel(
   const int pid = page_id(code);
   if (pid >= num_pages) return;
   const bool carry = compressed[b] != 0 && !page_is_last(code);
+  if (!carry && !write_cache) return;   // nothing to add and nothing to write back
   const int64_t sbase = (((int64_t)l * B + b) * Hkv) * (int64_t)NB * BS + (int64_t)j * BS;
   const int64_t cbase = l * c_sl + pid * c_sp;
   const int n = BS * Hkv;
@@ -38,7 +39,7 @@ __global__ __launch_bounds__(kThreads) void global_score_kernel(
       v = Elem<T>::rnd(method == ZP_ACTIVATE_MAX ? fmaxf(v, old) : v + old);
       Elem<T>::st(scores, si, v);
     }
-    Elem<T>::st(cache, cbase + c, v);
+    if (write_cache) Elem<T>::st(cache, cbase + c, v);
   }
 }
 
@@ -219,7 +220,7 @@ extern "C" int zp_global_score(void* scores, void* score_cache, const int32_t* b
                                const uint8_t* compressed, int32_t L, int32_t B, int32_t NB,
                                int32_t BS, int32_t Hkv, int32_t num_pages, int64_t c_sl,
                                int64_t c_sp, float decay_factor, int32_t activate_method,
-                               int32_t dtype, void* stream) {
+                               int32_t write_cache, int32_t dtype, void* stream) {
   ZP_REQUIRE(scores && score_cache && block_table && compressed, "global_score: null pointer");
   ZP_REQUIRE(L >= 0 && B >= 0 && NB > 0 && BS > 0 && Hkv > 0, "global_score: bad dims");
   ZP_REQUIRE(decay_factor >= 0.f && decay_factor <= 1.f, "global_score: decay_factor %g outside [0,1]",
@@ -232,7 +233,7 @@ extern "C" int zp_global_score(void* scores, void* score_cache, const int32_t* b
   ZP_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((global_score_kernel<T>), grid, dim3(kThreads), 0, st,
                                               scores, score_cache, block_table, compressed, B, NB,
                                               BS, Hkv, num_pages, c_sl, c_sp, decay_factor,
-                                              activate_method));
+                                              activate_method, write_cache));
   ZP_LAUNCH_CHECK();
   return ZP_OK;
 }

@@ -8,8 +8,14 @@ _METHODS = {"max": 0, "sum": 1}
 
 def global_score(reduced_scores: torch.Tensor, score_cache: torch.Tensor,
                  block_table: torch.Tensor, compressed: torch.Tensor,
-                 decay_factor: float = 0.9, activate_method: str = "max") -> torch.Tensor:
+                 decay_factor: float = 0.9, activate_method: str = "max", *,
+                 write_cache: bool = True) -> torch.Tensor:
     """max(new, old*decay) (or the sum) against the carried score cache.
+
+    ``write_cache=False`` (not in the reference) leaves the score cache untouched: the reference
+    stores every sequence's result into its pages (global_score.py:73-74), which races when
+    sequences of one batch share prefix pages; the carried values are then compacted from the
+    returned scores (``compress_score(..., scores_src=...)``).
 
     reduced_scores: (L, B, Hkv, NB, BS), updated in place and returned; score_cache:
     (L, num_pages, BS, Hkv), updated in place; block_table: (B, NB) int32; compressed:
@@ -30,6 +36,6 @@ def global_score(reduced_scores: torch.Tensor, score_cache: torch.Tensor,
     _lib.call("zp_global_score", _lib.dev_ptr(reduced_scores), _lib.dev_ptr(score_cache),
               _lib.dev_ptr(block_table), _lib.dev_ptr(compressed), L, B, NB, BS, Hkv, num_pages,
               score_cache.stride(0), score_cache.stride(1), float(decay_factor),
-              _METHODS[activate_method], _lib.dtype_tag(reduced_scores),
+              _METHODS[activate_method], int(write_cache), _lib.dtype_tag(reduced_scores),
               _lib.stream_ptr(reduced_scores))
     return reduced_scores
