@@ -194,6 +194,70 @@ int zp_compress_score(void* score_cache, const void* scores_src, const uint8_t* 
                       int64_t c_stride_layer, int64_t c_stride_page, int64_t c_stride_slot,
                       int64_t c_stride_head, int32_t dtype, void* stream);
 
+/* ---- one layer chunk of the compression step as one call ----
+ * The body of ModelRunner.compress for one chunk of layers
+ * (zipage/engine/model_runner.py:466-622): attention_score -> [max-norm, global_score] ->
+ * [redundancy] -> pooling / combine / sink / window mask / pad mask / top-k -> compress_kv ->
+ * [compress_score], enqueued on `stream` in that order by the entry points above, so every
+ * result is bit-identical to calling them one after the other.  The switches are the fields of
+ * zipage/config.py:22-46 that the runner reads. */
+typedef struct {
+  int32_t budget_blocks;          /* max_cache_blocks_per_seq: k = BS * budget_blocks survive */
+  int32_t query_cache_len;        /* window W (also the window mask) */
+  float softmax_scale;            /* <= 0: head_dim^-1/2 */
+  int32_t reduced;                /* ZP_REDUCE_* */
+  int32_t use_global_score;
+  float decay_factor;
+  int32_t activate_method;        /* ZP_ACTIVATE_* */
+  int32_t max_norm;
+  int32_t use_redundancy;
+  int32_t lightning;              /* 1: per page, 0: all pairs */
+  double redundancy_lambda;
+  double redundancy_temperature;
+  float redundancy_threshold;
+  int32_t pooling_size;           /* <= 1: no pooling */
+  int32_t continues_pooling;
+  int32_t pooling_mode;           /* ZP_POOL_* */
+  int32_t sink_len;               /* 0: no attention sink */
+  int32_t deterministic_carry;    /* see zp_global_score: 1 = carried scores come from the
+                                     scores, no shared page is written; 0 = the reference */
+} zp_compress_config;
+
+/* Stage names of the reference's timers (zipage/engine/model_runner.py:424-429,624-630);
+ * ZP_STAGE_SELECT is pooling + window_mask + topk_mask as the one launch this library uses
+ * when a row fits in LDS. */
+enum {
+  ZP_STAGE_ATTENTION_SCORE = 0, ZP_STAGE_GLOBAL_SCORE, ZP_STAGE_POOLING, ZP_STAGE_REDUNDANCY,
+  ZP_STAGE_WINDOW_MASK, ZP_STAGE_TOPK_MASK, ZP_STAGE_SELECT, ZP_STAGE_COMPRESS_KV,
+  ZP_STAGE_COMPRESS_SCORE, ZP_NUM_STAGES
+};
+
+/* Bytes of device workspace zp_compress_layers needs for these dims (scores, redundancy, the
+ * stages' own scratch, and the keep flags when flag_in_workspace != 0); -1 on bad arguments. */
+int64_t zp_compress_layers_workspace(int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
+                                     int32_t Hq, int32_t W, int32_t dtype,
+                                     const zp_compress_config* cfg, int32_t flag_in_workspace);
+
+/* k_cache / v_cache (L, num_pages, BS, Hkv, D), compacted in place; query_cache
+ * (L, max_seqs, W, Hq, D); score_cache (L, num_pages, BS, Hkv) or NULL (required with
+ * use_global_score), updated in place; seq_idx (B,) rows of the query cache; block_table
+ * (B, NB); compressed (B,) bytes; target_block_table (B, target_width); flag_out NULL or
+ * (L, B, Hkv, NB, BS) bytes receiving the keep flags.
+ * strides: 14 int64 element strides: key layer, page, slot, head; value layer, page, slot,
+ * head; query layer, sequence; score cache layer, page, slot, head (the last four ignored
+ * without a score cache).  workspace: 256-byte aligned, zp_compress_layers_workspace() bytes;
+ * its contents before the call do not matter and nothing in it is needed afterwards.
+ * stage_events: NULL, or a HOST array of 2 * ZP_NUM_STAGES hipEvent_t (start, stop per stage,
+ * NULL entries skipped) recorded on `stream` around the stages that run. */
+int zp_compress_layers(void* k_cache, void* v_cache, const void* query_cache, void* score_cache,
+                       const int32_t* seq_idx, const int32_t* block_table,
+                       const uint8_t* compressed, const int32_t* target_block_table,
+                       uint8_t* flag_out, int32_t L, int32_t B, int32_t NB, int32_t BS,
+                       int32_t Hkv, int32_t Hq, int32_t D, int32_t W, int32_t num_pages,
+                       int32_t max_seqs, int32_t target_width, const int64_t* strides,
+                       int32_t dtype, const zp_compress_config* cfg, void* workspace,
+                       int64_t workspace_bytes, void* const* stage_events, void* stream);
+
 /* ---- decode-step neighbours of the compression path (the callers either side of it) ---- */
 
 /* store_kvcache(key, value, k_cache, v_cache, slot_mapping)

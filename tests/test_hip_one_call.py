@@ -1,0 +1,81 @@
+"""zp_compress_layers (one host call per layer chunk, caller-passed workspace) against the same
+stages issued one entry point at a time: keep flags, K, V and the score cache must be the same
+bits, for every switch set the runner has (zipage/engine/model_runner.py:466-622)."""
+import pytest
+import torch
+
+from tests import cases
+
+pytestmark = pytest.mark.gpu
+
+SWITCHES = {
+    "pooling": dict(enable_pooling=True, pooling_size=7),
+    "plain": dict(),
+    "scripts": dict(use_global_score=True, decay_factor=0.8, enable_pooling=True,
+                    use_redudancy=True, lightning_redudancy=True),
+    "raw+sink+maxnorm": dict(use_global_score=True, max_norm=True, use_redudancy=True,
+                             lightning_redudancy=False, use_attention_sink=True, sink_len=4,
+                             enable_pooling=True, continues_pooling=True, pooling_mode="avg",
+                             activate_method="sum", decay_factor=0.9, redudancy_lambda=0.5),
+    "max-reduced": dict(reduced="max", enable_pooling=True),
+}
+
+
+def _inputs(dtype, seed=91, L=2, B=4, Hkv=2, Hq=8, W=16, budget=2):
+    tables, enc, target = cases.random_tables(seed, B, 40, [3, 4], budget)
+    k, v, q, sc = cases.make_caches(seed, L, 40, 256, Hkv, Hq, 128, W, B + 1, dtype,
+                                    touched=cases.touched_pages(enc), with_score_cache=True)
+    base = torch.randn((1, 1, 1, Hkv, 128), generator=torch.Generator().manual_seed(seed + 1))
+    k = (k.float() * 0.8 + 0.6 * base).to(dtype)
+    qid = torch.arange(B, dtype=torch.int32)
+    comp = torch.tensor([False, True, False, True][:B])
+    return k, v, q, sc, qid, enc, comp, target
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("name", list(SWITCHES))
+@pytest.mark.parametrize("deterministic_carry", [True, False])
+def test_one_call_equals_separate_stages(dev, dtype, name, deterministic_carry):
+    from zipage_amd.compress import CompressConfig, StageTimer, compress_layers
+    kw = SWITCHES[name]
+    if not kw.get("use_global_score") and not deterministic_carry:
+        pytest.skip("the carried-score mode only matters with the global score on")
+    k, v, q, sc, qid, enc, comp, target = _inputs(dtype)
+    cfg = CompressConfig(budget_blocks=2, query_cache_len=16, **kw)
+    outs = []
+    for one_call in (True, False):
+        gk, gv, gsc = k.clone().to(dev), v.clone().to(dev), sc.clone().to(dev)
+        timer = StageTimer(True)
+        res = compress_layers(gk, gv, q.to(dev), gsc, qid.to(dev), enc.to(dev), comp.to(dev),
+                              target.to(dev), cfg, timer=timer, return_intermediates=not one_call,
+                              deterministic_carry=deterministic_carry)
+        torch.cuda.synchronize()
+        flag = res if one_call else res[0]
+        secs = timer.seconds()
+        want = {"attention_score", "pooling+window_mask+topk_mask", "compress_kv"}
+        if kw.get("use_global_score"):
+            want |= {"global_score", "compress_global_score"}
+        if kw.get("use_redudancy"):
+            want.add("redudancy_score")
+        assert set(secs) == want and all(0 < s < 1 for s in secs.values()), secs
+        outs.append((flag.cpu(), gk.cpu(), gv.cpu(), gsc.cpu()))
+    for a, b in zip(*outs):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+    assert (outs[0][0].flatten(3).sum(-1) == 2 * 256).all()
+
+
+def test_one_call_rejects_a_short_workspace(dev):
+    import ctypes
+    from zipage_amd import _lib
+    from zipage_amd.compress import CompressConfig, c_config, layer_chunk_args
+    k, v, q, sc, qid, enc, comp, target = (t.to(dev) for t in _inputs(torch.bfloat16))
+    dims, strides = layer_chunk_args(k, v, q, sc, qid, enc, comp, target)
+    cc = c_config(CompressConfig(budget_blocks=2, query_cache_len=16))
+    lib = _lib.load()
+    need = lib.zp_compress_layers_workspace(*dims[:6], dims[7], 0, ctypes.byref(cc), 1)
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    with pytest.raises(RuntimeError, match="workspace of"):
+        _lib.call("zp_compress_layers", k.data_ptr(), v.data_ptr(), q.data_ptr(), 0, qid.data_ptr(),
+                  enc.data_ptr(), comp.data_ptr(), target.data_ptr(), 0, *dims, strides, 0,
+                  ctypes.byref(cc), ws.data_ptr(), need - 256, None, 0)

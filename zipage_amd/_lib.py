@@ -51,7 +51,29 @@ SIGNATURES = {
     "zp_qk_norm_rope_store": [ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, ptr, i32, i32,
                               i32, i32, i32, i64, i64, i32, i32, i64, i64, f32, i32, ptr],
 }
+
+
+class CompressConfigC(C.Structure):
+    """zp_compress_config of include/zipage_hip.h."""
+    _fields_ = [("budget_blocks", i32), ("query_cache_len", i32), ("softmax_scale", f32),
+                ("reduced", i32), ("use_global_score", i32), ("decay_factor", f32),
+                ("activate_method", i32), ("max_norm", i32), ("use_redundancy", i32),
+                ("lightning", i32), ("redundancy_lambda", f64), ("redundancy_temperature", f64),
+                ("redundancy_threshold", f32), ("pooling_size", i32), ("continues_pooling", i32),
+                ("pooling_mode", i32), ("sink_len", i32), ("deterministic_carry", i32)]
+
+
+# stage order of the ZP_STAGE_* enum, under the names the reference's timers use
+# (zipage/engine/model_runner.py:424-429); the one-launch selection has its own name
+STAGE_NAMES = ("attention_score", "global_score", "pooling", "redudancy_score", "window_mask",
+               "topk_mask", "pooling+window_mask+topk_mask", "compress_kv", "compress_global_score")
+
+SIGNATURES["zp_compress_layers"] = (
+    [ptr] * 9 + [i32] * 11 + [C.POINTER(i64), i32, C.POINTER(CompressConfigC), ptr, i64,
+                              C.POINTER(ptr), ptr])
 I64_RETURNING = {
+    "zp_compress_layers_workspace": [i32, i32, i32, i32, i32, i32, i32, i32,
+                                     C.POINTER(CompressConfigC), i32],
     "zp_attention_score_workspace": [i32, i32, i32, i32, i32, i32, i32],
     "zp_redundancy_raw_workspace": [i32, i32, i32, i32, i32],
 }

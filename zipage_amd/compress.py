@@ -11,9 +11,12 @@ work whose result equals its input, so pooling is decided per sequence on the de
 """
 from __future__ import annotations
 
+import ctypes
 from dataclasses import dataclass
 
 import torch
+
+from zipage_amd import _lib
 
 from zipage_amd.kernel.attention_score import attention_score
 from zipage_amd.kernel.compress_kv import compress_kv
@@ -79,6 +82,22 @@ class StageTimer:
         if ed is not None:
             ed.record()
 
+    def event_array(self, stages):
+        """Start / stop event handles for ``zp_compress_layers`` (a host array of
+        2 * ZP_NUM_STAGES hipEvent_t; stages that are not timed stay NULL), or None."""
+        if not self.enabled:
+            return None
+        arr = (ctypes.c_void_p * (2 * len(_lib.STAGE_NAMES)))()
+        for i, name in enumerate(_lib.STAGE_NAMES):
+            if name not in stages or (self.only is not None and name not in self.only):
+                continue
+            st, ed = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            st.record()   # torch creates the HIP event on its first record
+            ed.record()
+            arr[2 * i], arr[2 * i + 1] = st.cuda_event, ed.cuda_event
+            self.spans.append((name, st, ed))
+        return arr
+
     def seconds(self):
         """Per-stage totals; call after the stream has been synchronised."""
         out = {}
@@ -108,6 +127,10 @@ def compress_layers(k_cache, v_cache, query_cache, score_cache, query_ids, block
     """
     t = timer or StageTimer(False)
     BS = k_cache.shape[2]
+    if fused_select and not return_intermediates and block_tables.shape[1] * BS <= MAX_ROW_TOKENS:
+        return _compress_layers_one_call(k_cache, v_cache, query_cache, score_cache, query_ids,
+                                         block_tables, compressed, target_block_tables, cfg, t,
+                                         deterministic_carry)
 
     ev = t.start("attention_score")
     scores = attention_score(k_cache, query_cache, query_ids, block_tables, cfg.softmax_scale,
@@ -178,4 +201,85 @@ def compress_layers(k_cache, v_cache, query_cache, score_cache, query_ids, block
         t.stop(ev)
     if return_intermediates:
         return flag, scores
+    return flag
+
+
+_REDUCE = {"mean": 0, "max": 1}
+_ACTIVATE = {"max": 0, "sum": 1}
+_POOL = {"max": 0, "avg": 1}
+
+
+def c_config(cfg: CompressConfig, deterministic_carry=True) -> "_lib.CompressConfigC":
+    if cfg.reduced not in _REDUCE:
+        raise ValueError(f"Invalid reduction method: {cfg.reduced}")
+    assert cfg.activate_method in _ACTIVATE and cfg.pooling_mode in _POOL
+    assert 0 <= cfg.decay_factor <= 1
+    return _lib.CompressConfigC(
+        budget_blocks=cfg.budget_blocks, query_cache_len=cfg.query_cache_len,
+        softmax_scale=-1.0 if cfg.softmax_scale is None else float(cfg.softmax_scale),
+        reduced=_REDUCE[cfg.reduced], use_global_score=int(cfg.use_global_score),
+        decay_factor=float(cfg.decay_factor), activate_method=_ACTIVATE[cfg.activate_method],
+        max_norm=int(cfg.max_norm), use_redundancy=int(cfg.use_redudancy),
+        lightning=int(cfg.lightning_redudancy), redundancy_lambda=float(cfg.redudancy_lambda),
+        redundancy_temperature=float(cfg.redudancy_temperature),
+        redundancy_threshold=float(cfg.redudancy_threshold),
+        pooling_size=cfg.pooling_size if cfg.enable_pooling else 0,
+        continues_pooling=int(cfg.continues_pooling), pooling_mode=_POOL[cfg.pooling_mode],
+        sink_len=cfg.sink_len if cfg.use_attention_sink else 0,
+        deterministic_carry=int(deterministic_carry))
+
+
+def layer_chunk_args(k_cache, v_cache, query_cache, score_cache, query_ids, block_tables,
+                     compressed, target_block_tables):
+    """Shape checks and the dims / strides block shared by the one-call entry points."""
+    L, num_pages, BS, Hkv, D = k_cache.shape
+    _, max_seqs, W, Hq, _ = query_cache.shape
+    B, NB = block_tables.shape
+    assert v_cache.shape == k_cache.shape and v_cache.dtype == k_cache.dtype
+    assert query_cache.shape[0] == L and query_cache.dtype == k_cache.dtype
+    assert query_cache.is_contiguous() and k_cache.stride(4) == 1 and v_cache.stride(4) == 1
+    assert query_ids.shape == (B,) and query_ids.dtype == torch.int32 and query_ids.is_contiguous()
+    assert block_tables.dtype == torch.int32 and block_tables.is_contiguous()
+    assert compressed.shape == (B,) and compressed.dtype == torch.bool
+    assert target_block_tables.shape[0] == B and target_block_tables.dtype == torch.int32
+    assert target_block_tables.is_contiguous()
+    strides = list(k_cache.stride()[:4]) + list(v_cache.stride()[:4]) + list(query_cache.stride()[:2])
+    if score_cache is not None:
+        assert score_cache.shape == (L, num_pages, BS, Hkv) and score_cache.dtype == k_cache.dtype
+        strides += list(score_cache.stride())
+    else:
+        strides += [0, 0, 0, 0]
+    dims = (L, B, NB, BS, Hkv, Hq, D, W, num_pages, max_seqs, target_block_tables.shape[1])
+    return dims, (ctypes.c_int64 * 14)(*strides)
+
+
+def _compress_layers_one_call(k_cache, v_cache, query_cache, score_cache, query_ids, block_tables,
+                              compressed, target_block_tables, cfg, timer, deterministic_carry):
+    """The whole chunk through ``zp_compress_layers``: one host call enqueues every stage; the
+    only allocations are the keep flags and the workspace (torch's caching allocator)."""
+    dims, strides = layer_chunk_args(k_cache, v_cache, query_cache, score_cache, query_ids,
+                                     block_tables, compressed, target_block_tables)
+    L, B, NB, BS, Hkv, Hq, D, W = dims[:8]
+    if cfg.use_global_score:
+        assert score_cache is not None
+    flag = torch.empty((L, B, Hkv, NB, BS), device=k_cache.device, dtype=torch.bool)
+    if flag.numel() == 0:
+        return flag
+    cc = c_config(cfg, deterministic_carry)
+    lib = _lib.load()
+    tag = _lib.dtype_tag(k_cache)
+    ws_bytes = lib.zp_compress_layers_workspace(L, B, NB, BS, Hkv, Hq, W, tag, ctypes.byref(cc), 0)
+    ws = torch.empty(ws_bytes, device=k_cache.device, dtype=torch.uint8)
+    running = {"attention_score", FUSED_SELECT_STAGE, "compress_kv"}
+    if cfg.use_global_score:
+        running |= {"global_score", "compress_global_score"}
+    if cfg.use_redudancy:
+        running.add("redudancy_score")
+    events = timer.event_array(running)
+    compressed = compressed.contiguous()
+    _lib.call("zp_compress_layers", _lib.dev_ptr(k_cache), _lib.dev_ptr(v_cache),
+              _lib.dev_ptr(query_cache), _lib.dev_ptr(score_cache), _lib.dev_ptr(query_ids),
+              _lib.dev_ptr(block_tables), _lib.dev_ptr(compressed),
+              _lib.dev_ptr(target_block_tables), _lib.dev_ptr(flag), *dims, strides, tag,
+              ctypes.byref(cc), _lib.dev_ptr(ws), ws_bytes, events, _lib.stream_ptr(k_cache))
     return flag
