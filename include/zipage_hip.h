@@ -258,6 +258,26 @@ int zp_compress_layers(void* k_cache, void* v_cache, const void* query_cache, vo
                        int32_t dtype, const zp_compress_config* cfg, void* workspace,
                        int64_t workspace_bytes, void* const* stage_events, void* stream);
 
+/* The same call for callers that cannot allocate device memory -- code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.
+ * The workspace is a fixed array of ZP_STATIC_SCRATCH_BYTES in device memory that the library
+ * owns (one per GPU, held until the process ends), so the call takes no workspace and calls no
+ * hipMalloc / hipFree or allocating routine; flag_out may be NULL (the flags then live in the
+ * array too).  A chunk whose zp_compress_layers_workspace() exceeds the array is refused with
+ * ZP_EINVAL: 32 MiB covers one layer of 256 sequences x 10 pages at 8 kv heads in a 16-bit
+ * dtype with the lightning redundancy on.  Every call on a GPU uses that GPU's one array: calls
+ * that overlap in time on one GPU (two streams, two threads) race and must be serialised by the
+ * caller.  Nothing in the array has to be cleared between calls. */
+#define ZP_STATIC_SCRATCH_BYTES (32u << 20)
+int zp_compress_layers_static(void* k_cache, void* v_cache, const void* query_cache,
+                              void* score_cache, const int32_t* seq_idx,
+                              const int32_t* block_table, const uint8_t* compressed,
+                              const int32_t* target_block_table, uint8_t* flag_out, int32_t L,
+                              int32_t B, int32_t NB, int32_t BS, int32_t Hkv, int32_t Hq,
+                              int32_t D, int32_t W, int32_t num_pages, int32_t max_seqs,
+                              int32_t target_width, const int64_t* strides, int32_t dtype,
+                              const zp_compress_config* cfg, void* stream);
+
 /* ---- decode-step neighbours of the compression path (the callers either side of it) ---- */
 
 /* store_kvcache(key, value, k_cache, v_cache, slot_mapping)

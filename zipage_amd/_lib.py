@@ -71,6 +71,9 @@ STAGE_NAMES = ("attention_score", "global_score", "pooling", "redudancy_score", 
 SIGNATURES["zp_compress_layers"] = (
     [ptr] * 9 + [i32] * 11 + [C.POINTER(i64), i32, C.POINTER(CompressConfigC), ptr, i64,
                               C.POINTER(ptr), ptr])
+SIGNATURES["zp_compress_layers_static"] = (
+    [ptr] * 9 + [i32] * 11 + [C.POINTER(i64), i32, C.POINTER(CompressConfigC), ptr])
+STATIC_SCRATCH_BYTES = 32 << 20
 I64_RETURNING = {
     "zp_compress_layers_workspace": [i32, i32, i32, i32, i32, i32, i32, i32,
                                      C.POINTER(CompressConfigC), i32],

@@ -4,7 +4,13 @@
 // workspace the caller passes in.  Nothing here launches a kernel of its own: each stage is the
 // entry point that also stands alone in this ABI, so results are bit-identical to calling them
 // one after the other.
+//
+// zp_compress_layers_static is the same call for callers that cannot allocate device memory
+// (code under HIP graph capture, tight serving loops): its workspace is a fixed array in device
+// memory that belongs to the library.
 #include "common.h"
+
+#include <mutex>
 
 namespace {
 
@@ -191,6 +197,36 @@ int check_dims(int L, int B, int NB, int BS, int Hkv, int Hq, int D, int W, int 
   return ZP_OK;
 }
 
+// ---- the library's own scratch: one array per GPU, in that GPU's memory, for the life of the
+// process.  Host code only ever uses the address hipGetSymbolAddress returns for it.
+static __device__ __align__(256) unsigned char scratch[ZP_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+char* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+int static_scratch(char** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    zp_set_error("compress_layers_static: no current device (%s)", hipGetErrorString(e));
+    return ZP_EHIP;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) {
+      zp_set_error("compress_layers_static: hipGetSymbolAddress failed on device %d: %s", dev,
+                   hipGetErrorString(e));
+      return ZP_EHIP;
+    }
+    g_scratch_ptr[dev] = (char*)ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return ZP_OK;
+}
+
 }  // namespace
 
 extern "C" int64_t zp_compress_layers_workspace(int32_t L, int32_t B, int32_t NB, int32_t BS,
@@ -226,4 +262,34 @@ extern "C" int zp_compress_layers(void* k_cache, void* v_cache, const void* quer
   return run_layers(k_cache, v_cache, query_cache, score_cache, seq_idx, block_table, compressed,
                     target_block_table, flag_out, L, B, NB, BS, Hkv, Hq, D, W, num_pages, max_seqs,
                     target_width, strides, dtype, cfg, (char*)workspace, p, stage_events, stream);
+}
+
+extern "C" int zp_compress_layers_static(void* k_cache, void* v_cache, const void* query_cache,
+                                         void* score_cache, const int32_t* seq_idx,
+                                         const int32_t* block_table, const uint8_t* compressed,
+                                         const int32_t* target_block_table, uint8_t* flag_out,
+                                         int32_t L, int32_t B, int32_t NB, int32_t BS,
+                                         int32_t Hkv, int32_t Hq, int32_t D, int32_t W,
+                                         int32_t num_pages, int32_t max_seqs,
+                                         int32_t target_width, const int64_t* strides,
+                                         int32_t dtype, const zp_compress_config* cfg,
+                                         void* stream) {
+  int rc = check_dims(L, B, NB, BS, Hkv, Hq, D, W, dtype);
+  if (rc != ZP_OK) return rc;
+  rc = check_config(cfg);
+  if (rc != ZP_OK) return rc;
+  ZP_REQUIRE(k_cache && v_cache && query_cache && seq_idx && block_table && compressed &&
+                 target_block_table && strides, "compress_layers_static: null pointer");
+  if (L == 0 || B == 0) return ZP_OK;
+  const Plan p = make_plan(L, B, NB, BS, Hkv, Hq, W, dtype, cfg, flag_out == nullptr);
+  ZP_REQUIRE(p.total <= (int64_t)ZP_STATIC_SCRATCH_BYTES,
+             "compress_layers_static: this chunk needs %lld bytes of scratch, the library's array "
+             "holds %lld; split the batch or the layers, or use zp_compress_layers with a "
+             "workspace", (long long)p.total, (long long)ZP_STATIC_SCRATCH_BYTES);
+  char* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc != ZP_OK) return rc;
+  return run_layers(k_cache, v_cache, query_cache, score_cache, seq_idx, block_table, compressed,
+                    target_block_table, flag_out, L, B, NB, BS, Hkv, Hq, D, W, num_pages, max_seqs,
+                    target_width, strides, dtype, cfg, ws, p, nullptr, stream);
 }
