@@ -288,19 +288,23 @@ def lightning_redudancy_score(key_cache, block_table, threshold=0.5, temperature
 
 
 def raw_redudancy_logits(key_cache, block_table, threshold=0.5, rounding="reference",
-                         col_chunk=16):
+                         col_chunk=16, return_partial_max=False):
     """Whole-sequence redundancy row sums ``(L,B,Hkv,NB*BS)`` (raw_redudancy_score.py:
     10-155,218-222).  Same rule as the lightning variant but the similarity matrix spans
     every cached key of the sequence; the diagonal is the global one (:107-111) and "last
     row" is by logical position because row pages are visited last to first (:84).
     The reference keeps one partial row sum per column page, accumulated in the cache
     dtype over that page's 16-column chunks (:146-155), then sums the partials over
-    column pages (:218); ``rounding="reference"`` follows that chain."""
+    column pages (:218); ``rounding="reference"`` follows that chain.
+    ``return_partial_max`` also returns, per key, the largest magnitude any of its partial sums
+    reached along the chain (tests size their tolerance by it: one fp32-order rounding flip
+    inside the chain moves the result by one unit in the last place of a PARTIAL sum)."""
     L, _, BS, Hkv, D = key_cache.shape
     B, NB = block_table.shape
     dt = key_cache.dtype
     norm = key_norm(key_cache, block_table)
     out = torch.full((L, B, Hkv, NB * BS), NEG_INF, dtype=torch.float32)
+    pmax = torch.zeros((L, B, Hkv, NB * BS), dtype=torch.float32)
     for b in range(B):
         valid = [j for j in range(NB) if int(block_table[b, j]) != -1]
         kh = torch.cat([
@@ -312,14 +316,20 @@ def raw_redudancy_logits(key_cache, block_table, threshold=0.5, rounding="refere
         sim = _claim_last_over_threshold(sim, threshold)
         if rounding == "fp32" or dt == torch.float32:
             rows = sim.sum(dim=-1)
+            big = rows.abs()
         else:
             chunks = sim.view(L, Hkv, Tv, len(valid), BS // col_chunk, col_chunk).sum(-1)
             part = torch.zeros((L, Hkv, Tv, len(valid)), dtype=torch.float32)
+            big = torch.zeros((L, Hkv, Tv), dtype=torch.float32)
             for c in range(BS // col_chunk):
                 part = _rnd(part + chunks[..., c], dt, rounding)
+                big = torch.maximum(big, part.abs().amax(dim=-1))
             rows = _rnd(part.sum(dim=-1), dt, rounding)
         for n, j in enumerate(valid):
             out[:, b, :, j * BS:(j + 1) * BS] = rows[:, :, n * BS:(n + 1) * BS]
+            pmax[:, b, :, j * BS:(j + 1) * BS] = big[:, :, n * BS:(n + 1) * BS]
+    if return_partial_max:
+        return out.to(dt), pmax
     return out.to(dt)
 
 

@@ -41,6 +41,26 @@ def test_prefix_sharing_refcounts_and_release():
     assert c.block_table[:4] == d.block_table[:4] and c.block_table[4] != d.block_table[4]
 
 
+def test_a_fully_cached_prompt_still_prefills_its_last_page():
+    """Two identical prompts of exactly two pages: every page of the second one hits the prefix
+    cache, but its last page is taken fresh so that prefill runs the last prompt token (the
+    first decode step feeds on it) instead of decoding from a stale token."""
+    pool = PagePool(16, 16, pages_per_seq=5, enable_prefix_cache=True)
+    a, b = _seq(32), _seq(32)
+    pool.admit(a)
+    pool.admit(b)
+    assert a.block_table[0] == b.block_table[0] and a.block_table[1] != b.block_table[1]
+    assert b.num_cached_tokens == 16 < len(b)
+    cfg = EngineConfig(shape=TINY, max_concurrency=4, num_kvcache_blocks=16, kvcache_block_size=16,
+                       max_cache_blocks_per_seq=4, enable_prefix_cache=True)
+    sched = Scheduler(cfg)
+    x, y = _seq(32), _seq(32)
+    sched.add(x)
+    sched.add(y)
+    batch, is_prefill = sched.schedule()
+    assert is_prefill and batch == [x, y], "both prompts must go through prefill"
+
+
 @pytest.mark.parametrize("seed", range(6))
 def test_plan_compression_follows_the_copy_on_write_rule(seed):
     """Against the oracle's restatement of BlockManager.may_compress on random sharing patterns."""

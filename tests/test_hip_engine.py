@@ -215,6 +215,17 @@ def test_prefix_cache_shares_pages_between_equal_prompts(dev):
     assert pool.num_free == cfg.num_kvcache_blocks and not pool.refcount.any()
 
 
+def test_identical_page_aligned_prompts_with_prefix_cache(dev):
+    """Two identical prompts of exactly one page with the prefix cache on: the second one must
+    produce the tokens of a run without sharing (a prompt whose every page hit the cache used to
+    skip prefill and decode from a stale token, overwriting the shared page)."""
+    prompt = _prompts(1, [256], seed=21)[0]
+    _, shared = _generate(_cfg(use_graph=False, enable_prefix_cache=True), [prompt, list(prompt)], 12)
+    _, solo = _generate(_cfg(use_graph=False), [prompt], 12)
+    assert shared[0]["token_ids"] == solo[0]["token_ids"]
+    assert shared[1]["token_ids"] == solo[0]["token_ids"]
+
+
 def test_reference_script_switches_through_the_engine(dev):
     """The switch set of the reference's scripts (global score with decay 0.8 and max-norm,
     lightning redundancy, pooling, attention sink) through the whole engine: the score cache is

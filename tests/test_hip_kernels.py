@@ -319,7 +319,7 @@ def test_redundancy_key_magnitudes(dev, dtype, scale, variant):
                                              temperature=0.4, return_logits=True)
     else:
         wl, wr = O.raw_redudancy_score(k, s["enc"], threshold=0.45, temperature=0.4,
-                                       return_logits=True, rounding="fp32")
+                                       return_logits=True)
         gl, gr = K.raw_redudancy_score(k.to(dev), s["enc"].to(dev), threshold=0.45,
                                        temperature=0.4, return_logits=True)
     _ulp_close(gl, wl, dtype, ulps=1, abs_floor=1e-2)
@@ -342,7 +342,7 @@ def test_redundancy_page_and_head_sizes(dev, dtype, BS, D, variant):
         wl, wr = O.lightning_redudancy_score(k, s["enc"], **kw)
         gl, gr = K.lightning_redudancy_score(k.to(dev), s["enc"].to(dev), **kw)
     else:
-        wl, wr = O.raw_redudancy_score(k, s["enc"], rounding="reference" if dtype == torch.float32 else "fp32", **kw)
+        wl, wr = O.raw_redudancy_score(k, s["enc"], **kw)
         gl, gr = K.raw_redudancy_score(k.to(dev), s["enc"].to(dev), **kw)
     if dtype == torch.float32:
         _rel_close(gl, wl, rel=1e-4, abs_floor=1e-2)
@@ -364,7 +364,7 @@ def test_raw_redundancy_page_counts(dev, dtype, nb_choices):
     k = (s["k"].float() * 0.7 + base).to(dtype)
     for thr in (0.35, 0.6):
         wl, wr = O.raw_redudancy_score(k, s["enc"], threshold=thr, temperature=0.4,
-                                       return_logits=True, rounding="fp32")
+                                       return_logits=True)
         gl, gr = raw_redudancy_score(k.to(dev), s["enc"].to(dev), threshold=thr, temperature=0.4,
                                      return_logits=True)
         _ulp_close(gl, wl, dtype, ulps=1, abs_floor=1e-2)
@@ -377,9 +377,8 @@ def test_raw_redundancy(dev, dtype):
     s = _setup(53, dtype, L=1, B=2, Hkv=2, Hq=2, nb_choices=(2, 3), num_pages=12)
     base = torch.randn((1, 1, 1, 2, 128), generator=torch.Generator().manual_seed(2))
     k = (s["k"].float() * 0.6 + base).to(dtype)
-    mode = "reference" if dtype == torch.float32 else "fp32"
     wl, wr = O.raw_redudancy_score(k, s["enc"], threshold=0.5, temperature=0.4,
-                                   return_logits=True, rounding=mode)
+                                   return_logits=True)
     gl, gr = raw_redudancy_score(k.to(dev), s["enc"].to(dev), threshold=0.5, temperature=0.4,
                                  return_logits=True)
     if dtype == torch.float32:

@@ -286,6 +286,70 @@ def test_raw_bruteforce_and_single_page_equals_lightning():
     assert torch.allclose(red[0, 0].reshape(Hkv, -1), torch.softmax(x, -1), atol=1e-6)
 
 
+def _raw_program_walk(e_pages, thr, dtype, block_m=64, block_n=16):
+    """The all-pairs kernel's own loop nest, one program per column page
+    (zipage/kernel/raw_redudancy_score.py:50-155), on normalised keys ``e_pages[page] (BS, D)``
+    fp32: columns in chunks of 16, row pages last to first, rows in blocks of 64 from the end; a
+    column is claimed by the first block row that exceeds the threshold in this order (:113-131);
+    the block's row sums are added to the column page's partial sums, which are kept in the
+    cache dtype (:133-155).  Then the partial sums of the column pages are added in fp32 and
+    rounded once (:218)."""
+    n_pages, BS = len(e_pages), e_pages[0].shape[0]
+    partial = torch.zeros((n_pages, n_pages, BS), dtype=dtype)       # [column page][row page]
+    ar = torch.arange(block_m).view(-1, 1)
+    for n in range(n_pages):
+        for n_off in range(0, BS, block_n):
+            cols = e_pages[n][n_off:n_off + block_n]
+            zo = torch.zeros((1, block_n), dtype=torch.bool)
+            for m in range(n_pages - 1, -1, -1):
+                for m_off in range(BS - block_m, -1, -block_m):
+                    sim = e_pages[m][m_off:m_off + block_m] @ cols.T
+                    if m == n:
+                        same = (m_off + ar) == (n_off + torch.arange(block_n).view(1, -1))
+                        sim = torch.where(same, torch.zeros_like(sim), sim)
+                    tm = (sim > thr) & ~zo
+                    last_idx = torch.where(tm, ar.expand_as(sim), torch.full_like(sim, -1, dtype=torch.long)).max(0, keepdim=True).values
+                    last = ar == last_idx
+                    sim = torch.where(last, torch.zeros_like(sim), sim)
+                    zo = zo | last.any(0, keepdim=True)
+                    cur = partial[n, m, m_off:m_off + block_m].float()
+                    partial[n, m, m_off:m_off + block_m] = (sim.sum(1) + cur).to(dtype)
+    return partial.float().sum(0).to(dtype)      # (row page, BS)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_raw_reference_rounding_chain(dtype):
+    """The oracle's restatement of the partial-sum chain (16-bit caches) against a literal walk
+    of the reference kernel's loop nest: same claims, same chain of cache-dtype roundings.  The
+    two add a chunk's 16 similarities in a different fp32 order, so a sum that lands on a rounding
+    boundary may differ by one unit in the last place; nothing else may."""
+    g = torch.Generator().manual_seed(12)
+    L, P, BS, Hkv, D = 1, 5, 64, 2, 8
+    base = torch.randn((1, 1, 1, Hkv, D), generator=g)
+    k = (torch.randn((L, P, BS, Hkv, D), generator=g) * 0.8 + 0.5 * base).to(dtype)
+    enc = torch.tensor([[3, 0, -6, -1], [1, -4, -1, -1]], dtype=torch.int32)   # pages 3,0,4 / 1,2
+    thr = 0.5
+    got = O.raw_redudancy_logits(k, enc, threshold=thr).view(L, 2, Hkv, 4, BS)
+    plain = O.raw_redudancy_logits(k, enc, threshold=thr, rounding="fp32").view(L, 2, Hkv, 4, BS)
+    norm = O.key_norm(k, enc)
+    tables = [[3, 0, 4], [1, 2]]
+    differs_from_plain = 0
+    for b, table in enumerate(tables):
+        for h in range(Hkv):
+            e = [k[0, pid, :, h].float() / norm[0, b, h, j].float().unsqueeze(-1)
+                 for j, pid in enumerate(table)]
+            want = _raw_program_walk(e, thr, dtype)
+            g_ = got[0, b, h, :len(table)].float()
+            w_ = want.float()
+            eps = 2.0 ** (-8 if dtype == torch.bfloat16 else -11)
+            assert ((g_ - w_).abs() <= 2 * eps * w_.abs() + 1e-6).all()
+            assert (g_ == w_).float().mean() >= 0.97
+            differs_from_plain += int((plain[0, b, h, :len(table)].float() != w_).sum())
+        assert torch.isinf(got[0, b, :, len(table):]).all()
+    # the chain is not a no-op: rounding once at the end gives other bits on many rows
+    assert differs_from_plain > 20
+
+
 # ------------------------------------------------------------------ a8/a9 closed forms
 def test_combine_sink_window_pad():
     g = torch.Generator().manual_seed(11)

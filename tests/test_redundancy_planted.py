@@ -173,7 +173,7 @@ def test_oracle_claims_the_planted_pairs(dtype, variant):
         assert len(claimed) >= len(pairs)
 
 
-def _close_in_ulps(got, want, dtype, ulps, frac_exact):
+def _close_in_ulps(got, want, dtype, ulps, frac_exact, chain_scale=None):
     g, w = got.float().cpu(), want.float().cpu()
     assert torch.equal(torch.isinf(g), torch.isinf(w))
     fin = torch.isfinite(w)
@@ -181,6 +181,11 @@ def _close_in_ulps(got, want, dtype, ulps, frac_exact):
     eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11}[dtype]
     # sums near zero are the remainder of cancelling terms: fp32 order noise floor
     tol = ulps * 2 * eps * torch.maximum(w.abs(), g.abs()) + 2e-5
+    if chain_scale is not None:
+        # the all-pairs variant rounds a running partial sum after every chunk: an fp32 sum on a
+        # rounding boundary there moves the result by one unit in the last place of the PARTIAL
+        # sum, which can be larger than the result; allow two such flips per row
+        tol = tol + 2 * 2 * eps * chain_scale.reshape(-1)[fin.reshape(-1)]
     err = (g - w).abs()
     worst = float((err / tol).max())
     same = float((g == w).float().mean())
@@ -197,6 +202,7 @@ def test_planted_pairs_against_oracle(dev, dtype, variant, thr):
     from zipage_amd import kernel as K
     k, enc, tables, plan = planted_case(103, dtype)
     kw = dict(threshold=thr, temperature=0.4, return_logits=True)
+    chain_scale = None
     if variant == "lightning":
         wl, wr = O.lightning_redudancy_score(k, enc, **kw)
         noclaim = O.lightning_redudancy_logits(k, enc, 2.0)
@@ -204,15 +210,19 @@ def test_planted_pairs_against_oracle(dev, dtype, variant, thr):
     else:
         wl, wr = O.raw_redudancy_score(k, enc, rounding=RAW_ORACLE_ROUNDING, **kw)
         noclaim = O.raw_redudancy_logits(k, enc, 2.0, rounding=RAW_ORACLE_ROUNDING)
+        chain_scale = O.raw_redudancy_logits(k, enc, thr, rounding=RAW_ORACLE_ROUNDING,
+                                             return_partial_max=True)[1]
         gl, gr = K.raw_redudancy_score(k.to(dev), enc.to(dev), **kw)
     if thr > 0:
         # the comparison is only worth something if claims moved many rows by far more than a ulp
         moved = ((noclaim.float().reshape(-1) - wl.float().reshape(-1)).abs() > 0.4)
         moved = moved & torch.isfinite(wl.float().reshape(-1))
         assert int(moved.sum()) >= 2 * 12 * HKV, f"only {int(moved.sum())} rows carry a claim"
-    _close_in_ulps(gl, wl, dtype, ulps=1, frac_exact=0.97)
+    _close_in_ulps(gl, wl, dtype, ulps=1, frac_exact=0.97,
+                   chain_scale=chain_scale if variant == "raw" else None)
     _close_in_ulps(gr, wr, dtype, ulps=4, frac_exact=0.5)
 
 
-# rounding chain of the all-pairs variant the GPU kernel is held to
-RAW_ORACLE_ROUNDING = "fp32"
+# rounding chain of the all-pairs variant the GPU kernel is held to: the reference's partial sums
+# in the cache dtype (zipage/kernel/raw_redudancy_score.py:146-155,218)
+RAW_ORACLE_ROUNDING = "reference"

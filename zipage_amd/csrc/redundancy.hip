@@ -18,8 +18,9 @@
 //                      split into two bf16 planes, three MFMAs per k-step, full matrix.
 //   gram_page_kernel   16-bit caches, lightning: stored keys on the matrix cores, 1/norm
 //                      factors on the accumulators, every pair of key blocks once.
-//   raw_rowsum_kernel, gram_raw_kernel, raw_claim_value_kernel
-//                      16-bit caches, raw: the same over the pages of a sequence.
+//   raw_prep_kernel, gram_raw_kernel, raw_claim_value_kernel, raw_chain_kernel
+//                      16-bit caches, raw: the same over the pages of a sequence, the row sums
+//                      accumulated in the cache dtype chunk by chunk as the reference does.
 //   red_softmax_kernel claim corrections of the raw variant and the softmax of both.
 #include "common.h"
 #include <math.h>
@@ -65,6 +66,8 @@ constexpr int TN = 64;                  // keys per column tile
 constexpr int ROWF = kDmax + 4;         // floats per LDS row: 16-byte aligned rows whose 16-byte reads by
                                         // eight consecutive rows fall into eight different bank groups
 constexpr int KS = kDmax / 2;           // MFMA k-steps (2 per instruction)
+constexpr int kChunk = 16;              // columns the reference's all-pairs kernel takes per step
+                                        // (BLOCK_N, raw_redudancy_score.py:176)
 
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -107,6 +110,7 @@ struct GramArgs {
   float* ws_sum;   // raw: fp32 plain row sums
   int32_t* ws_col; // raw: last column over the threshold (logical index, -1 none)
   float* ws_val;   // raw: its value
+  float* ws_chunk; // raw, 16-bit caches: [row][T / 16][kDmax] sums of the normalised keys per chunk
   int B, NB, BS, Hkv, D, num_pages;
   int64_t k_sl, k_sp;
   float threshold, eps;
@@ -980,69 +984,58 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
 }
 
 // ------------------------------------------------------------------ raw, 16-bit caches
-// All-pairs variant over the whole sequence.  Three launches share the symmetric scheme of the
-// page kernel above, with pages in the role of its 32-key blocks:
-//   1. raw_rowsum_kernel: one workgroup per (layer, sequence, head) sums the normalised keys of
-//      the sequence and writes every key's row sum  e_i . (S - e_i); claims start at "none".
+// All-pairs variant over the whole sequence.  Four launches; the claims use the symmetric scheme
+// of the page kernel above, with pages in the role of its 32-key blocks:
+//   1. raw_prep_kernel: 1 / norm of every key, the sum of the normalised keys of every 16-key
+//      chunk; claims start at "none".
 //   2. gram_raw_kernel: one workgroup per valid page a; it multiplies page a with the pages
 //      (a + d) mod n, d = 0..n/2, so every unordered pair of pages is done once, and records for
 //      the keys on both sides the last (logical) column over the threshold with integer
 //      atomic maxima (order-independent, so the result is deterministic).
 //   3. raw_claim_value_kernel: the fp32 value of every key's claimed entry.
-// The softmax kernel then subtracts the claimed values from the rows they were taken from.
+//   4. raw_chain_kernel: the row sums, accumulated chunk by chunk in the cache dtype as the
+//      reference does, with the diagonal and the claimed entries taken out of their chunks.
+// The softmax kernel then normalises the rows.
 
+// One workgroup per valid page: 1 / norm of every key, claims reset to "none", and the sum of the
+// normalised keys of every 16-key chunk of the page (fp32), which is all the row sums need:
+//   sum_{j in chunk} e_i . e_j = e_i . (sum_{j in chunk} e_j).
+// The reference walks the columns in chunks of 16 (BLOCK_N, raw_redudancy_score.py:176) and
+// rounds after each chunk, so the chunk is the unit whose sum has to be exact.
 template <typename T>
-__global__ __launch_bounds__(512) void raw_rowsum_kernel(GramArgs p) {
+__global__ __launch_bounds__(kThreads) void raw_prep_kernel(GramArgs p) {
   static_assert(T::bytes == 2, "16-bit caches only");
-  constexpr int kT = 512, PIECES = kDmax / 8, GROUPS = kT / PIECES, UNR = 4;
-  extern __shared__ __align__(16) char smem[];
-  float* l_part = (float*)smem;                       // [waves][kDmax]
-  int* vpage = (int*)(l_part + (kT / 64) * kDmax);
-  int* vidx = vpage + p.NB;
-  __shared__ int nvalid_s;
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int PIECES = kDmax / 8, GROUPS = kThreads / PIECES;   // 16 groups of 16 lanes
+  const int tid = threadIdx.x;
   const int piece = tid % PIECES, g = tid / PIECES;
-  const int h = blockIdx.x % p.Hkv;
-  const int b = (blockIdx.x / p.Hkv) % p.B;
-  const int l = blockIdx.x / (p.Hkv * p.B);
+  const int jp = blockIdx.x % p.NB;
+  const int h = (blockIdx.x / p.NB) % p.Hkv;
+  const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
+  const int l = blockIdx.x / (p.NB * p.Hkv * p.B);
   const int Tn = p.NB * p.BS;
-  const int64_t obase = (int64_t)blockIdx.x * Tn;
+  const int64_t obase = (((int64_t)l * p.B + b) * p.Hkv + h) * Tn + (int64_t)jp * p.BS;
   const float epsr = Elem<T>::rnd(p.eps);
-  if (tid == 0) {
-    int n = 0;
-    for (int j = 0; j < p.NB; ++j) {
-      const int c = p.table[(int64_t)b * p.NB + j];
-      const int pid = page_is_pad(c) ? -1 : page_id(c);
-      if (pid >= 0 && pid < p.num_pages) { vpage[n] = pid; vidx[n] = j; ++n; }
-    }
-    nvalid_s = n;
-  }
-  __syncthreads();
-  const int nrows = nvalid_s * p.BS;
-  const int dpieces = p.D / 8;
-  const bool pok = piece < dpieces;
+  const int code = p.table[(int64_t)b * p.NB + jp];
+  int rpid = page_is_pad(code) ? -1 : page_id(code);
+  if (rpid >= p.num_pages) rpid = -1;
+  if (rpid < 0) return;
+  const bool pok = piece < p.D / 8;
   const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
-  const char* kbase = p.k + (l * p.k_sl) * 2 + (int64_t)h * p.D * 2 + (pok ? piece : 0) * 16;
-  auto key_ptr = [&](int r) {
-    const int vp = r / p.BS, slot = r - vp * p.BS;
-    return kbase + (int64_t)vpage[vp] * p.k_sp * 2 + (int64_t)slot * k_row;
-  };
-
-  float cs[8];
+  const char* kbase = p.k + (l * p.k_sl + (int64_t)rpid * p.k_sp) * 2 + (int64_t)h * p.D * 2 +
+                      (pok ? piece : 0) * 16;
+  const int cpp = p.BS / kChunk;                       // chunks per page
+  float* csum = p.ws_chunk + (obase / kChunk) * kDmax;  // [chunk][kDmax] of this page
+  for (int c = g; c < cpp; c += GROUPS) {
+    u32x4 raw[kChunk];
 #pragma unroll
-  for (int q = 0; q < 8; ++q) cs[q] = 0.f;
-  for (int r0 = g; r0 < nrows; r0 += GROUPS * UNR) {
-    u32x4 raw[UNR];
+    for (int u = 0; u < kChunk; ++u)
+      raw[u] = *(const u32x4*)(kbase + (int64_t)(c * kChunk + u) * k_row);
+    float cs[8];
 #pragma unroll
-    for (int u = 0; u < UNR; ++u) {
-      const int r = r0 + u * GROUPS;
-      raw[u] = *(const u32x4*)key_ptr(r < nrows ? r : 0);
-    }
+    for (int q = 0; q < 8; ++q) cs[q] = 0.f;
 #pragma unroll
-    for (int u = 0; u < UNR; ++u) {
-      const bool ok = pok && r0 + u * GROUPS < nrows;
-      if (!ok) raw[u] = u32x4{0u, 0u, 0u, 0u};
+    for (int u = 0; u < kChunk; ++u) {
+      if (!pok) raw[u] = u32x4{0u, 0u, 0u, 0u};
       float e[8];
       Unpack<T>::run(vec16{raw[u].x, raw[u].y, raw[u].z, raw[u].w}, e);
       float ss = 0.f;
@@ -1052,59 +1045,16 @@ __global__ __launch_bounds__(512) void raw_rowsum_kernel(GramArgs p) {
       const float rn = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr));
 #pragma unroll
       for (int q = 0; q < 8; ++q) cs[q] = fmaf(e[q], rn, cs[q]);
+      if (piece == 0) {
+        const int64_t oi = obase + c * kChunk + u;
+        p.ws_sum[oi] = rn;      // kept for the row-sum kernel
+        p.ws_val[oi] = rn;      // read by the Gram kernel, replaced by the claim values after it
+        p.ws_col[oi] = -1;
+      }
     }
-  }
-#pragma unroll
-  for (int q = 0; q < 8; ++q) {
-    cs[q] += lane_xor16(cs[q]);
-    cs[q] += lane_xor32(cs[q]);
-  }
-  if (lane < PIECES) {
-    float* dst = l_part + wave * kDmax + piece * 8;
+    float* dst = csum + (int64_t)c * kDmax + piece * 8;
     *(float4*)dst = make_float4(cs[0], cs[1], cs[2], cs[3]);
     *(float4*)(dst + 4) = make_float4(cs[4], cs[5], cs[6], cs[7]);
-  }
-  __syncthreads();
-  float sv[8];
-#pragma unroll
-  for (int q = 0; q < 8; ++q) sv[q] = 0.f;
-#pragma unroll
-  for (int w = 0; w < kT / 64; ++w) {
-    const float* src = l_part + w * kDmax + piece * 8;
-    const float4 a = *(const float4*)src, c = *(const float4*)(src + 4);
-    sv[0] += a.x; sv[1] += a.y; sv[2] += a.z; sv[3] += a.w;
-    sv[4] += c.x; sv[5] += c.y; sv[6] += c.z; sv[7] += c.w;
-  }
-  for (int r0 = g; r0 < nrows; r0 += GROUPS * UNR) {
-    u32x4 raw[UNR];
-#pragma unroll
-    for (int u = 0; u < UNR; ++u) {
-      const int r = r0 + u * GROUPS;
-      raw[u] = *(const u32x4*)key_ptr(r < nrows ? r : 0);
-    }
-#pragma unroll
-    for (int u = 0; u < UNR; ++u) {
-      const int r = r0 + u * GROUPS;
-      if (!pok) raw[u] = u32x4{0u, 0u, 0u, 0u};
-      float e[8];
-      Unpack<T>::run(vec16{raw[u].x, raw[u].y, raw[u].z, raw[u].w}, e);
-      float ss = 0.f, t = 0.f;
-#pragma unroll
-      for (int q = 0; q < 8; ++q) {
-        ss = fmaf(e[q], e[q], ss);
-        t = fmaf(e[q], sv[q], t);
-      }
-      ss = pieces_sum<PIECES>(ss);
-      t = pieces_sum<PIECES>(t);
-      const float rn = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr));
-      if (piece == 0 && r < nrows) {
-        const int vp = r / p.BS, slot = r - vp * p.BS;
-        const int64_t oi = obase + (int64_t)vidx[vp] * p.BS + slot;
-        p.ws_sum[oi] = t * rn - ss * rn * rn;
-        p.ws_col[oi] = -1;
-        p.ws_val[oi] = rn;      // read by the Gram kernel, replaced by the claim values after it
-      }
-    }
   }
 }
 
@@ -1172,7 +1122,7 @@ void gram_raw_kernel(GramArgs p) {
   const int dpieces = p.D / 8;
   const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
   const char* kbase = p.k + (l * p.k_sl) * 2 + (int64_t)h * p.D * 2;
-  const float* rn_all = p.ws_val + obase;           // written by raw_rowsum_kernel
+  const float* rn_all = p.ws_val + obase;           // written by raw_prep_kernel
 
   const int st_piece = tid % PIECES, st_row0 = tid / PIECES;
   const bool st_ok = st_piece < dpieces;
@@ -1376,6 +1326,185 @@ __global__ __launch_bounds__(kThreads) void raw_claim_value_kernel(GramArgs p) {
   }
 }
 
+// ------------------------------------------------------------------ raw, 16-bit: row sums
+// The reference accumulates a key's row sum in the CACHE dtype: per column page one partial sum,
+// rounded after each 16-column chunk (raw_redudancy_score.py:146-155: load, add the chunk's fp32
+// sum, store in the cache dtype), then the partial sums of the pages are added in fp32 and rounded
+// once (:218, torch.sum).  This kernel restates that chain exactly.
+//   chunk sum   c(i, chunk) = rn_i (k_i . s_chunk) - [i in chunk] S_ii - sum_{j in chunk, claimed by i} S_ij
+// with s_chunk the sum of the chunk's normalised keys from raw_prep_kernel.  The dot products of
+// a page's 256 keys with 32 chunks at a time run on the matrix cores: the keys as stored (exact
+// 16-bit products), s_chunk split into three 16-bit planes (together its full fp32 mantissa).
+// One workgroup per valid page; wave w owns keys 32 w .. 32 w + 31.
+template <typename T> struct Split3;
+template <> struct Split3<BF16> {
+  __device__ static __forceinline__ void run(float v, uint16_t* o) {
+    const float h = bf16_round(v), m = bf16_round(v - h), l = bf16_round(v - h - m);
+    o[0] = (uint16_t)(__float_as_uint(h) >> 16);
+    o[1] = (uint16_t)(__float_as_uint(m) >> 16);
+    o[2] = (uint16_t)(__float_as_uint(l) >> 16);
+  }
+};
+template <> struct Split3<F16> {
+  __device__ static __forceinline__ void run(float v, uint16_t* o) {
+    o[0] = float_to_f16_bits(v);
+    const float r1 = v - f16_bits_to_float(o[0]);
+    o[1] = float_to_f16_bits(r1);
+    o[2] = float_to_f16_bits(r1 - f16_bits_to_float(o[1]));
+  }
+};
+// chunk sums are below 16 + 1 in magnitude: 2^-26 fixed point fits 32 bits, and integer atomics
+// make the sum of several claims independent of their order
+__device__ __forceinline__ int to_fixed26(float v) { return (int)(v * 67108864.f); }
+__device__ __forceinline__ float from_fixed26(int w) { return (float)w * (1.f / 67108864.f); }
+
+template <typename T>
+__global__ __launch_bounds__(512) void raw_chain_kernel(GramArgs p) {
+  static_assert(T::bytes == 2, "16-bit caches only");
+  typedef typename Mfma16<T>::V frag_t;
+  constexpr int kT = 512, kW = 8, KSB = kDmax / 16, CT = 32;     // CT chunks per tile
+  constexpr int KEYS = kW * 32;                                     // keys per round
+  extern __shared__ __align__(16) char smem[];
+  char* planes = smem;                                   // [3][CT] rows of ROWH bytes
+  int* cl = (int*)(smem + 3 * CT * ROWH);                // [CT][KEYS] corrections, then chunk sums
+  int* vidx = cl + CT * KEYS;                            // [NB] logical page of the n-th valid page
+  int* vord = vidx + p.NB;                               // [NB] inverse (-1: pad)
+  __shared__ int nvalid_s;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const int jp = blockIdx.x % p.NB;
+  const int h = (blockIdx.x / p.NB) % p.Hkv;
+  const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
+  const int l = blockIdx.x / (p.NB * p.Hkv * p.B);
+  const int Tn = p.NB * p.BS;
+  const int64_t obase = (((int64_t)l * p.B + b) * p.Hkv + h) * Tn;
+
+  const int code = p.table[(int64_t)b * p.NB + jp];
+  int rpid = page_is_pad(code) ? -1 : page_id(code);
+  if (rpid >= p.num_pages) rpid = -1;
+  if (rpid < 0) {
+    for (int s = tid; s < p.BS; s += kT) Elem<T>::st(p.r_out, obase + (int64_t)jp * p.BS + s, -INFINITY);
+    return;
+  }
+  if (tid == 0) {
+    int n = 0;
+    for (int j = 0; j < p.NB; ++j) {
+      const int c = p.table[(int64_t)b * p.NB + j];
+      const int pid = page_is_pad(c) ? -1 : page_id(c);
+      if (pid >= 0 && pid < p.num_pages) { vidx[n] = j; vord[j] = n; ++n; } else vord[j] = -1;
+    }
+    nvalid_s = n;
+  }
+  __syncthreads();
+  const int cpp = p.BS / kChunk;
+  const int nchunks = nvalid_s * cpp;
+  const int ntiles = (nchunks + CT - 1) / CT;
+  const int my_ord = vord[jp];
+  const int dpieces = p.D / 8;
+  const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
+  const char* kpage = p.k + (l * p.k_sl + (int64_t)rpid * p.k_sp) * 2 + (int64_t)h * p.D * 2;
+  const float* chunk_all = p.ws_chunk + (obase / kChunk) * kDmax;
+
+  const int rounds = (p.BS + KEYS - 1) / KEYS;
+  for (int rr = 0; rr < rounds; ++rr) {
+    const int key0 = rr * KEYS;                       // first slot of this round
+    const int slot = key0 + wave * 32 + col;          // this lane's key (both halves of the wave)
+    const bool live = slot < p.BS;
+    // ---- B fragments: the key as stored; lane (key, half) holds k = 16 s + 8 half + i
+    frag_t bk[KSB];
+    float ssq = 0.f;
+    {
+      const char* src = kpage + (int64_t)(live ? slot : 0) * k_row;
+#pragma unroll
+      for (int s = 0; s < KSB; ++s) {
+        const int pc = 2 * s + half;
+        u32x4 v = u32x4{0u, 0u, 0u, 0u};
+        if (live && pc < dpieces) v = *(const u32x4*)(src + pc * 16);
+        bk[s] = __builtin_bit_cast(frag_t, v);
+        float e[8];
+        Unpack<T>::run(vec16{v.x, v.y, v.z, v.w}, e);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) ssq = fmaf(e[q], e[q], ssq);
+      }
+      ssq += lane_xor32(ssq);
+    }
+    const float rn = live ? p.ws_sum[obase + (int64_t)jp * p.BS + slot] : 0.f;
+    const float diag = ssq * rn * rn;                 // S_ii, the entry the reference zeroes
+    const int own_chunk = my_ord * cpp + slot / kChunk;
+    float part = 0.f, total = 0.f;                    // chain state of key `tid` (tid < KEYS)
+
+    for (int tile = 0; tile < ntiles; ++tile) {
+      const int c0 = tile * CT;
+      // ---- corrections of this tile, and its three planes
+      for (int i = tid; i < CT * KEYS; i += kT) cl[i] = 0;
+      for (int i = tid; i < CT * (kDmax / 4); i += kT) {
+        const int m = i / (kDmax / 4), q4 = i - m * (kDmax / 4);
+        const int vc = c0 + m;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (vc < nchunks) {
+          const int vp = vc / cpp, c = vc - vp * cpp;
+          v = *(const float4*)(chunk_all + ((int64_t)vidx[vp] * cpp + c) * kDmax + q4 * 4);
+        }
+        const float f[4] = {v.x, v.y, v.z, v.w};
+        uint16_t o[4][3];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) Split3<T>::run(f[q], o[q]);
+#pragma unroll
+        for (int pl = 0; pl < 3; ++pl) {
+          uint2 w;
+          w.x = (uint32_t)o[0][pl] | ((uint32_t)o[1][pl] << 16);
+          w.y = (uint32_t)o[2][pl] | ((uint32_t)o[3][pl] << 16);
+          *(uint2*)(planes + (pl * CT + m) * ROWH + q4 * 8) = w;
+        }
+      }
+      __syncthreads();
+      if (half == 0 && live && own_chunk >= c0 && own_chunk < c0 + CT)
+        atomicAdd(&cl[(own_chunk - c0) * KEYS + wave * 32 + col], to_fixed26(diag));
+      for (int t = tid; t < Tn; t += kT) {
+        const int jt = t / p.BS;
+        const int ord = vord[jt];
+        if (ord < 0) continue;
+        const int vc = ord * cpp + (t - jt * p.BS) / kChunk;
+        if (vc < c0 || vc >= c0 + CT) continue;
+        const int cc = p.ws_col[obase + t] - (jp * p.BS + key0);   // the row key t claimed from
+        if (cc >= 0 && cc < KEYS && key0 + cc < p.BS)
+          atomicAdd(&cl[(vc - c0) * KEYS + cc], to_fixed26(p.ws_val[obase + t]));
+      }
+      __syncthreads();
+      // ---- chunk sums of the tile: A = planes (rows = chunks), B = keys
+      {
+        f32x16_t acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+        for (int pl = 2; pl >= 0; --pl) {
+          const char* arow = planes + (pl * CT + col) * ROWH + half * 16;
+#pragma unroll
+          for (int s = 0; s < KSB; ++s) acc = Mfma16<T>::run(*(const frag_t*)(arow + s * 32), bk[s], acc);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int m = (r >> 2) * 8 + half * 4 + (r & 3);
+          int* slot_p = &cl[m * KEYS + wave * 32 + col];
+          *slot_p = __float_as_int(acc[r] * rn - from_fixed26(*slot_p));
+        }
+      }
+      __syncthreads();
+      // ---- the reference's chain: one cache-dtype partial sum per column page
+      if (tid < KEYS) {
+        for (int m = 0; m < CT && c0 + m < nchunks; ++m) {
+          if ((c0 + m) % cpp == 0) { total += part; part = 0.f; }
+          part = Elem<T>::rnd(part + __int_as_float(cl[m * KEYS + tid]));
+        }
+      }
+      __syncthreads();
+    }
+    if (tid < KEYS && key0 + tid < p.BS)
+      Elem<T>::st(p.r_out, obase + (int64_t)jp * p.BS + key0 + tid, total + part);
+  }
+}
+
 // ------------------------------------------------------------------ softmax epilogue
 // One workgroup per (layer, sequence, head) row of T logits:
 //   raw only: r_i = rowsum_i - sum_{j: c*(j)=i} v_j, pad pages -inf
@@ -1396,13 +1525,15 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
     void* __restrict__ red, void* __restrict__ logits, const int32_t* __restrict__ table,
     const float* __restrict__ ws_sum, const int32_t* __restrict__ ws_col,
     const float* __restrict__ ws_val, int B, int NB, int BS, int Hkv, int num_pages,
-    float tscale /* raw: temperature; lightning: temperature*BS */) {
+    float tscale /* raw: temperature; lightning: temperature*BS */,
+    int rows_ready /* raw: the row sums are already in `red` (16-bit caches) */) {
   extern __shared__ __align__(16) char smem[];
   __shared__ float red_lds[kWaves];
   const int Tn = NB * BS;
   // raw: [Tn] 64-bit sums of the values claimed from each row, then the [Tn] floats of the row
   unsigned long long* corr = (unsigned long long*)smem;
-  float* x = (float*)(smem + (RAW ? (size_t)Tn * 8 : 0));
+  const bool from_ws = RAW && !rows_ready;
+  float* x = (float*)(smem + (from_ws ? (size_t)Tn * 8 : 0));
   const int64_t row = blockIdx.x;
   const int b = (int)((row / Hkv) % B);
   const int64_t base = row * Tn;
@@ -1414,7 +1545,7 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
     nvalid += (pid >= 0 && pid < num_pages) ? 1 : 0;
   }
   const float divisor = RAW ? tscale * (float)(nvalid * BS) : tscale;
-  if (RAW) {
+  if (from_ws) {
     // every key hands the value of its claimed entry to the row it was taken from: 2^-32 fixed
     // point with integer atomics, exact and independent of the order
     for (int t = threadIdx.x; t < Tn; t += kThreads) corr[t] = 0ull;
@@ -1431,7 +1562,7 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
   float mloc = -INFINITY;
   for (int t = threadIdx.x; t < Tn; t += kThreads) {
     float r;
-    if (RAW) {
+    if (from_ws) {
       const int c = trow[t / BS];
       const int pid = page_is_pad(c) ? -1 : page_id(c);
       if (pid >= 0 && pid < num_pages) {
@@ -1511,21 +1642,23 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
     }
   }
   if constexpr (T::bytes == 2 && RAW) {
-    const size_t smem0 = (size_t)(512 / 64) * kDmax * 4 + sizeof(int) * 2 * a.NB;
     // column tiles of 128 keys when the page size allows: half as many workgroup barriers
     const int tn = a.BS % 128 == 0 ? 128 : TN;
     const size_t smem1 = 2 * (size_t)tn * ROWH + sizeof(int) * 4 * tn + sizeof(float) * a.BS +
                          sizeof(int) * 2 * a.NB;
     const void* fn = tn == 128 ? (const void*)gram_raw_kernel<T, 128> : (const void*)gram_raw_kernel<T, TN>;
-    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1) != hipSuccess) {
-      zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem1);
+    const size_t smem2 = 3 * 32 * (size_t)ROWH + sizeof(int) * 32 * 256 + sizeof(int) * 2 * a.NB;
+    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1) != hipSuccess ||
+        hipFuncSetAttribute((const void*)raw_chain_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)smem2) != hipSuccess) {
+      zp_set_error("redundancy: cannot reserve %zu / %zu bytes of LDS", smem1, smem2);
       return ZP_EHIP;
     }
-    hipLaunchKernelGGL((raw_rowsum_kernel<T>), dim3((unsigned)((int64_t)L * a.B * a.Hkv)), dim3(512),
-                       smem0, st, a);
+    hipLaunchKernelGGL((raw_prep_kernel<T>), grid, dim3(kThreads), 0, st, a);
     if (tn == 128) hipLaunchKernelGGL((gram_raw_kernel<T, 128>), grid, dim3(512), smem1, st, a);
     else hipLaunchKernelGGL((gram_raw_kernel<T, TN>), grid, dim3(512), smem1, st, a);
     hipLaunchKernelGGL((raw_claim_value_kernel<T>), grid, dim3(kThreads), 0, st, a);
+    hipLaunchKernelGGL((raw_chain_kernel<T>), grid, dim3(512), smem2, st, a);
     ZP_LAUNCH_CHECK();
     return ZP_OK;
   }
@@ -1561,8 +1694,8 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
 template <typename T, bool RAW>
 int launch_softmax(void* red, void* logits, const int32_t* table, const float* ws_sum,
                    const int32_t* ws_col, const float* ws_val, int L, int B, int NB, int BS,
-                   int Hkv, int num_pages, double temperature, hipStream_t st) {
-  const size_t smem = (size_t)NB * BS * (RAW ? 12 : 4);
+                   int Hkv, int num_pages, double temperature, hipStream_t st, int rows_ready = 0) {
+  const size_t smem = (size_t)NB * BS * ((RAW && !rows_ready) ? 12 : 4);
   if (smem > 150 * 1024) {
     zp_set_error("redundancy: a row of %d tokens exceeds LDS", NB * BS);
     return ZP_EUNSUPPORTED;
@@ -1576,7 +1709,7 @@ int launch_softmax(void* red, void* logits, const int32_t* table, const float* w
   dim3 grid((unsigned)((int64_t)L * B * Hkv));
   hipLaunchKernelGGL((red_softmax_kernel<T, RAW>), grid, dim3(kThreads), smem, st, red, logits,
                      table, ws_sum, ws_col, ws_val, B, NB, BS, Hkv, num_pages,
-                     RAW ? (float)temperature : (float)(temperature * (double)BS));
+                     RAW ? (float)temperature : (float)(temperature * (double)BS), rows_ready);
   ZP_LAUNCH_CHECK();
   return ZP_OK;
 }
@@ -1595,7 +1728,7 @@ extern "C" int zp_redundancy_lightning(const void* k_cache, const int32_t* block
   if (L == 0 || B == 0) return ZP_OK;
   GramArgs a;
   a.k = (const char*)k_cache; a.table = block_table; a.r_out = red_out;
-  a.ws_sum = nullptr; a.ws_col = nullptr; a.ws_val = nullptr;
+  a.ws_sum = nullptr; a.ws_col = nullptr; a.ws_val = nullptr; a.ws_chunk = nullptr;
   a.B = B; a.NB = NB; a.BS = BS; a.Hkv = Hkv; a.D = D; a.num_pages = num_pages;
   a.k_sl = k_sl; a.k_sp = k_sp; a.threshold = threshold; a.eps = 1e-6f;
   hipStream_t st = (hipStream_t)stream;
@@ -1610,7 +1743,8 @@ extern "C" int zp_redundancy_lightning(const void* k_cache, const int32_t* block
 
 extern "C" int64_t zp_redundancy_raw_workspace(int32_t L, int32_t B, int32_t NB, int32_t BS,
                                                int32_t Hkv) {
-  return (int64_t)L * B * Hkv * NB * BS * 12;
+  // three fp32 / int32 words per key, and for 16-bit caches kDmax floats per chunk of 16 keys
+  return (int64_t)L * B * Hkv * NB * BS * (12 + 4 * kDmax / kChunk);
 }
 
 extern "C" int zp_redundancy_raw(const void* k_cache, const int32_t* block_table, void* red_out,
@@ -1623,12 +1757,15 @@ extern "C" int zp_redundancy_raw(const void* k_cache, const int32_t* block_table
   if (rc != ZP_OK) return rc;
   if (L == 0 || B == 0) return ZP_OK;
   const int64_t n = (int64_t)L * B * Hkv * NB * BS;
-  ZP_REQUIRE(workspace && workspace_bytes >= n * 12,
-             "redundancy_raw: workspace of %lld bytes required", (long long)n * 12);
-  ZP_REQUIRE(((uintptr_t)workspace % 4) == 0, "redundancy_raw: workspace must be 4-byte aligned");
+  const int64_t need = zp_redundancy_raw_workspace(L, B, NB, BS, Hkv);
+  ZP_REQUIRE(workspace && workspace_bytes >= need,
+             "redundancy_raw: workspace of %lld bytes required", (long long)need);
+  ZP_REQUIRE(((uintptr_t)workspace % 16) == 0, "redundancy_raw: workspace must be 16-byte aligned");
   GramArgs a;
-  a.k = (const char*)k_cache; a.table = block_table; a.r_out = nullptr;
+  a.k = (const char*)k_cache; a.table = block_table;
+  a.r_out = red_out;   // 16-bit caches: the row sums go here before the softmax
   a.ws_sum = (float*)workspace; a.ws_col = (int32_t*)workspace + n; a.ws_val = (float*)workspace + 2 * n;
+  a.ws_chunk = (float*)workspace + 3 * n;
   a.B = B; a.NB = NB; a.BS = BS; a.Hkv = Hkv; a.D = D; a.num_pages = num_pages;
   a.k_sl = k_sl; a.k_sp = k_sp; a.threshold = threshold; a.eps = 1e-6f;
   hipStream_t st = (hipStream_t)stream;
@@ -1636,7 +1773,7 @@ extern "C" int zp_redundancy_raw(const void* k_cache, const int32_t* block_table
     rc = launch_gram<T, true>(a, L, st);
     if (rc != ZP_OK) return rc;
     rc = launch_softmax<T, true>(red_out, logits_out, block_table, a.ws_sum, a.ws_col, a.ws_val, L,
-                                 B, NB, BS, Hkv, num_pages, temperature, st);
+                                 B, NB, BS, Hkv, num_pages, temperature, st, T::bytes == 2);
   });
   return rc;
 }

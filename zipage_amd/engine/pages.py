@@ -79,8 +79,10 @@ class PagePool:
 
     def admit(self, seq: Sequence):
         """Pages for a prompt; leading full pages already cached under the same chain hash are
-        shared (block_manager.py:78-112).  The last page of a prompt that already fills a whole
-        table is never shared: its window queries must be captured by running it."""
+        shared (block_manager.py:78-112).  The last page of a prompt is never shared: a prompt
+        whose every page hits would skip prefill altogether, and the first decode step needs the
+        last prompt token run through the model (and, when the prompt fills a whole table, the
+        window queries of that page captured)."""
         assert not seq.block_table
         h, miss = -1, False
         for i in range(seq.num_blocks):
@@ -88,8 +90,7 @@ class PagePool:
             full = len(toks) == self.page_size and self.enable_prefix_cache
             h = self.chain_hash(toks, h) if full else -1
             page = self.by_hash.get(h, -1)
-            holds_window = i == seq.num_blocks - 1 and seq.num_blocks >= self.pages_per_seq
-            if page == -1 or self.page_tokens[page] != toks or holds_window:
+            if page == -1 or self.page_tokens[page] != toks or i == seq.num_blocks - 1:
                 miss = True
             if miss:
                 page = self._take()
