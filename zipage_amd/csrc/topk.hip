@@ -1,10 +1,9 @@
 // Per-row top-k keep mask by radix select (one workgroup per row).
 //
-// Scores are mapped to order-preserving 32-bit keys held in LDS.  The k-th largest key
-// v* is found most-significant-bit first: a candidate bit is kept when at least k keys
-// are >= the candidate prefix; each step is one block-wide count (ballot-free register
-// counts, xor-shuffle wave sums, one barrier with ping-pong LDS slots).  16-bit inputs
-// only need the upper 16 (bf16) or 19 (fp16) bits.  Every key > v* is kept; of the keys
+// Scores are mapped to order-preserving 32-bit keys.  The k-th largest key v* is found by a
+// radix select over 8-bit digits, most significant first (block_radix_select: LDS digit
+// histograms, a wave-level suffix scan over the bins, one barrier per pass); 16-bit inputs
+// only need the upper 16 (bf16: two passes) or 19 (fp16: three) bits.  Every key > v* is kept; of the keys
 // equal to v*, the k - count(>v*) with the LOWEST indices are kept, which a block-wide
 // exclusive scan over index-ordered per-thread chunks decides.
 #include "common.h"
@@ -13,6 +12,7 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
+constexpr int kHistCopies = 8;   // copies of the radix-select digit bins (see block_radix_select)
 
 // `low_bit`: the float image of this dtype has all bits below it clear; the key keeps them
 // clear too (for negatives the complement would set them), so the bit search can stop there.
@@ -24,14 +24,80 @@ __device__ __forceinline__ uint32_t score_key(float f, int low_bit) {
   return ((u & 0x80000000u) ? ~u : (u | 0x80000000u)) & keep;
 }
 
-__device__ __forceinline__ int block_count(int c, int* slots /* kWaves */) {
-  c = wave_sum_i(c);
-  if (lane_id() == 0) slots[wave_id()] = c;
-  __syncthreads();
-  int s = 0;
+// k-th largest key of a row held by the 256 threads of a workgroup, by radix select: 8 bits per
+// pass, most significant digit first.  Every thread adds the digit of each of its keys that still
+// matches the prefix to a 256-bin LDS histogram (fire-and-forget adds, no dependent chain); every
+// wave then reads the bins (four per lane), finds the bin that holds the k-th largest key with a
+// suffix scan over its lanes, and the search descends into that bin.  All waves compute the same
+// digit from the same bins, so one barrier per pass suffices (the bins rotate through three
+// buffers: the one cleared during a pass was last read two passes ago, with a barrier between).  bf16 keys take two passes,
+// fp16 three, fp32 four.  `each(f)` calls f(key) for every key of the calling thread.
+// Returns the k-th largest key; `n_gt` receives the number of keys strictly above it.
+template <typename Each>
+__device__ __forceinline__ uint32_t block_radix_select(Each each, int k, int low_bit, int* hist /* [3][kHistCopies][256] */,
+                                                       int& n_gt) {
+  const int tid = threadIdx.x, lane = tid & 63;
+  uint32_t prefix = 0;
+  int kk = k;
+  n_gt = 0;
+  if (k <= 0) return 0xffffffffu;            // above every key: nothing is kept
+  constexpr int HB = kHistCopies * 256;
 #pragma unroll
-  for (int i = 0; i < kWaves; ++i) s += slots[i];
-  return s;
+  for (int c = 0; c < kHistCopies; ++c) hist[c * 256 + tid] = 0;   // kThreads == 256 bins
+  __syncthreads();
+  int pp = 0;
+  // scores cluster in a few exponents, so most lanes of a wave hit the same few bins and LDS adds
+  // to one address serialise: lane l adds to copy l % kHistCopies of the bins
+  int* mycopy = hist + (lane % kHistCopies) * 256;
+  for (int sh = 24; sh + 8 > low_bit; sh -= 8) {
+    int* cur = hist + pp * HB;
+    const int nx = pp == 2 ? 0 : pp + 1;
+#pragma unroll
+    for (int c = 0; c < kHistCopies; ++c)
+      hist[nx * HB + c * 256 + tid] = 0;     // the next pass's bins (last read two passes ago)
+    const uint32_t hi_mask = sh == 24 ? 0u : (0xffffffffu << (sh + 8));
+    each([&](uint32_t key) {
+      if ((key & hi_mask) == prefix) atomicAdd(&mycopy[pp * HB + ((key >> sh) & 0xff)], 1);
+    });
+    __syncthreads();
+    int4 bins = *(const int4*)(cur + 4 * lane);
+#pragma unroll
+    for (int c = 1; c < kHistCopies; ++c) {
+      const int4 o = *(const int4*)(cur + c * 256 + 4 * lane);
+      bins.x += o.x; bins.y += o.y; bins.z += o.z; bins.w += o.w;
+    }
+    const int mine = bins.x + bins.y + bins.z + bins.w;
+    int suf = mine;                          // inclusive suffix sum over the lanes (higher digits)
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int t = __shfl_down(suf, o, 64);
+      if (lane + o < 64) suf += t;
+    }
+    const int above = suf - mine;            // keys in the bins of higher lanes
+    const bool here = above < kk && kk <= suf;
+    int digit = 0, over = 0;
+    if (here) {
+      const int bv[4] = {bins.x, bins.y, bins.z, bins.w};
+      int acc = above;
+      digit = -1;
+#pragma unroll
+      for (int q = 3; q >= 0; --q) {
+        if (digit < 0) {
+          if (acc + bv[q] >= kk) { digit = 4 * lane + q; over = acc; }
+          else acc += bv[q];
+        }
+      }
+    }
+    const unsigned long long who = __builtin_amdgcn_ballot_w64(here);
+    const int src = who ? __builtin_ctzll(who) : 0;   // exactly one lane when k <= row length
+    digit = __builtin_amdgcn_readlane(digit, src);
+    over = __builtin_amdgcn_readlane(over, src);
+    prefix |= (uint32_t)digit << sh;
+    n_gt += over;
+    kk -= over;
+    pp = nx;
+  }
+  return prefix;
 }
 
 template <typename T>
@@ -39,27 +105,17 @@ __global__ __launch_bounds__(kThreads) void topk_mask_kernel(const void* __restr
                                                              uint8_t* __restrict__ flag, int Tn,
                                                              int k, int low_bit) {
   extern __shared__ uint32_t keys[];
-  __shared__ int slots[2][kWaves];
+  __shared__ __align__(16) int hist[3][kHistCopies][256];
   __shared__ int scan_lds[kWaves];
   const int tid = threadIdx.x;
   const int64_t base = (int64_t)blockIdx.x * Tn;
   for (int t = tid; t < Tn; t += kThreads) keys[t] = score_key(Elem<T>::ld(scores, base + t), low_bit);
   __syncthreads();
 
-  uint32_t prefix = 0;
-  int pp = 0;
-  for (int bit = 31; bit >= low_bit; --bit) {
-    const uint32_t cand = prefix | (1u << bit);
-    int c = 0;
-    for (int t = tid; t < Tn; t += kThreads) c += keys[t] >= cand ? 1 : 0;
-    if (block_count(c, slots[pp]) >= k) prefix = cand;
-    pp ^= 1;
-  }
-  // keys strictly above the threshold
-  int cg = 0;
-  for (int t = tid; t < Tn; t += kThreads) cg += keys[t] > prefix ? 1 : 0;
-  const int n_gt = block_count(cg, slots[pp]);
-  const int need_eq = k - n_gt;  // >= 1 whenever k <= Tn
+  int n_gt;
+  const uint32_t prefix = block_radix_select(
+      [&](auto f) { for (int t = tid; t < Tn; t += kThreads) f(keys[t]); }, k, low_bit, &hist[0][0][0], n_gt);
+  const int need_eq = k - n_gt;  // >= 1 whenever 1 <= k <= Tn
 
   // index-ordered pass
   const int chunk = (Tn + kThreads - 1) / kThreads;
@@ -179,7 +235,7 @@ constexpr int kSelHalf = 3;
 template <typename T, int PER>
 __global__ __launch_bounds__(kThreads) void select_reg_kernel(SelectArgs p) {
   extern __shared__ float row[];
-  __shared__ int slots[2][kWaves];
+  __shared__ __align__(16) int hist[3][kHistCopies][256];
   __shared__ int scan_lds[kWaves];
   __shared__ float max_lds[kWaves];
   const int tid = threadIdx.x;
@@ -246,24 +302,18 @@ __global__ __launch_bounds__(kThreads) void select_reg_kernel(SelectArgs p) {
     }
   }
 
-  uint32_t prefix = 0;
-  int pp = 0;
-  for (int bit = 31; bit >= p.low_bit; --bit) {
-    const uint32_t cand = prefix | (1u << bit);
-    int c = 0;
+  int n_gt;
+  const uint32_t prefix = block_radix_select(
+      [&](auto f) {
 #pragma unroll
-    for (int i = 0; i < PER; ++i) c += kreg[i] >= cand ? 1 : 0;
-    if (block_count(c, slots[pp]) >= p.k) prefix = cand;
-    pp ^= 1;
-  }
+        for (int i = 0; i < PER; ++i) f(kreg[i]);
+      },
+      p.k, p.low_bit, &hist[0][0][0], n_gt);
   // prefix is the k-th largest key; keep everything above it and the first few equal to it
-  int cg = 0, ce = 0;
+  const int need_eq = p.k - n_gt;
+  int ce = 0;
 #pragma unroll
-  for (int i = 0; i < PER; ++i) {
-    cg += kreg[i] > prefix ? 1 : 0;
-    ce += (s0 + i < s1 && kreg[i] == prefix) ? 1 : 0;
-  }
-  const int need_eq = p.k - block_count(cg, slots[pp]);
+  for (int i = 0; i < PER; ++i) ce += (s0 + i < s1 && kreg[i] == prefix) ? 1 : 0;
   int inc = ce;
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) {
@@ -291,7 +341,7 @@ __global__ __launch_bounds__(kThreads) void select_reg_kernel(SelectArgs p) {
 template <typename T>
 __global__ __launch_bounds__(kThreads) void select_lds_kernel(SelectArgs p) {
   extern __shared__ float row[];
-  __shared__ int slots[2][kWaves];
+  __shared__ __align__(16) int hist[3][kHistCopies][256];
   __shared__ int scan_lds[kWaves];
   __shared__ float max_lds[kWaves];
   const int tid = threadIdx.x;
@@ -335,21 +385,12 @@ __global__ __launch_bounds__(kThreads) void select_lds_kernel(SelectArgs p) {
 
   const int chunk = (Tn + kThreads - 1) / kThreads;
   const int s0 = min(tid * chunk, Tn), s1 = min(s0 + chunk, Tn);
-  uint32_t prefix = 0;
-  int pp = 0;
-  for (int bit = 31; bit >= p.low_bit; --bit) {
-    const uint32_t cand = prefix | (1u << bit);
-    int c = 0;
-    for (int s = s0; s < s1; ++s) c += keys[s] >= cand ? 1 : 0;
-    if (block_count(c, slots[pp]) >= p.k) prefix = cand;
-    pp ^= 1;
-  }
-  int cg = 0, ce = 0;
-  for (int s = s0; s < s1; ++s) {
-    cg += keys[s] > prefix ? 1 : 0;
-    ce += keys[s] == prefix ? 1 : 0;
-  }
-  const int need_eq = p.k - block_count(cg, slots[pp]);
+  int n_gt;
+  const uint32_t prefix = block_radix_select(
+      [&](auto f) { for (int s = s0; s < s1; ++s) f(keys[s]); }, p.k, p.low_bit, &hist[0][0][0], n_gt);
+  const int need_eq = p.k - n_gt;
+  int ce = 0;
+  for (int s = s0; s < s1; ++s) ce += keys[s] == prefix ? 1 : 0;
   int inc = ce;
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) {
