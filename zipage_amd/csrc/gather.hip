@@ -18,9 +18,7 @@
 namespace {
 
 constexpr int kThreads = 256;
-#ifndef ZP_COMPACT_R
-#define ZP_COMPACT_R 8
-#endif
+constexpr int kCompactR = 8;   // 16-byte pieces each thread gathers per round
 // native vector types keep the staged pieces in VGPRs
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -67,12 +65,8 @@ struct CompactArgs {
 // Survivors are written once and not read again by this kernel: non-temporal stores keep them
 // from displacing the gather's source lines in L2 (measured at 256 sequences on one allocation:
 // 704 -> 686 us per launch; non-temporal loads on top: 720 us).
-#ifndef ZP_NT_LOAD
 #define ZP_NT_LOAD(ptr) (*(ptr))
-#endif
-#ifndef ZP_NT_STORE
 #define ZP_NT_STORE(v, ptr) __builtin_nontemporal_store(v, ptr)
-#endif
 // POW2: page size and pieces-per-vector are powers of two, so every index split is a shift.
 template <typename P, int R, bool HAS_B, bool POW2>
 __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
@@ -253,7 +247,7 @@ extern "C" int zp_compress_kv(void* key, void* value, const uint8_t* flag,
   ZP_REQUIRE((int64_t)target_width * BS * a.lpv < (int64_t)1 << 31, "compress_kv: row too large");
   hipStream_t st = (hipStream_t)stream;
   switch (piece) {
-    case 16: return launch_compact<u32x4, ZP_COMPACT_R, true>(a, L, st);
+    case 16: return launch_compact<u32x4, kCompactR, true>(a, L, st);
     case 8:  return launch_compact<u32x2, 8, true>(a, L, st);
     case 4:  return launch_compact<uint32_t, 8, true>(a, L, st);
     default: return launch_compact<uint16_t, 8, true>(a, L, st);

@@ -28,24 +28,14 @@
 
 namespace {
 
-#ifndef ZP_SCORE_WAVES
-#define ZP_SCORE_WAVES 4
-#endif
-constexpr int kWaves = ZP_SCORE_WAVES;  // waves per workgroup (4 or 8)
-#ifndef ZP_SCORE_TN16
-#define ZP_SCORE_TN16 (32 * kWaves)     // tokens per K tile for 16-bit caches
-#endif
-#ifndef ZP_SCORE_OCC
-#define ZP_SCORE_OCC 2                  // workgroups per CU the 16-bit kernel is compiled for
-#endif
+constexpr int kWaves = 4;               // waves per workgroup
+constexpr int kTN16 = 32 * kWaves;      // tokens per K tile for 16-bit caches
+constexpr int kOcc16 = 2;               // workgroups per CU the 16-bit kernel is compiled for
 constexpr int kThreads = kWaves * 64;
 constexpr int kRowWaves = 4;   // most waves along the query-row axis; the other factor splits tokens.
                                // Fewer row blocks (small window x group) use 2 or 1 row waves so
                                // that no wave idles: ScoreArgs::RW.
 constexpr int kDmax = 128;
-#ifndef ZP_SCORE_ZIGZAG
-#define ZP_SCORE_ZIGZAG 1
-#endif
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
@@ -54,14 +44,14 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 template <typename T> struct Mma;
 template <> struct Mma<BF16> {
   typedef bf16x8_t Frag;
-  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = ZP_SCORE_TN16, ROWB = kDmax * 2 + 16;
+  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = kTN16, ROWB = kDmax * 2 + 16;
   __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
 };
 template <> struct Mma<F16> {
   typedef f16x8_t Frag;
-  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = ZP_SCORE_TN16, ROWB = kDmax * 2 + 16;
+  static constexpr int KPI = 16, EPL = 8, KS = kDmax / KPI, TN = kTN16, ROWB = kDmax * 2 + 16;
   __device__ static __forceinline__ f32x16_t mma(Frag a, Frag b, f32x16_t c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
@@ -104,9 +94,6 @@ template <> struct Rnd<F32> {
 };
 template <> struct Rnd<BF16> {
   __device__ static __forceinline__ void pair(float& a, float& b) {
-#ifdef ZP_DBG_NORND
-    return;
-#endif
     // v_cvt_pk_bf16_f32 with a zero in the low half: the 32-bit result IS the rounded value as
     // fp32, so each value costs one instruction and nothing has to be unpacked
     typedef __attribute__((ext_vector_type(2))) float f2;
@@ -139,17 +126,11 @@ __device__ __forceinline__ float vmax_neg(float a, float b) {  // max(a, -b)
 
 // exp of a non-positive argument, natural base, via the hardware base-2 exponential.
 __device__ __forceinline__ float exp_neg(float x) {
-#ifdef ZP_DBG_NOEXP
-  return x * 1.44269504088896340736f;
-#endif
   return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
 }
 
 // 2^y through the hardware exponential (y <= 0 here; -inf gives 0).
 __device__ __forceinline__ float exp2_hw(float y) {
-#ifdef ZP_DBG_NOEXP
-  return y;
-#endif
   return __builtin_amdgcn_exp2f(y);
 }
 
@@ -158,7 +139,7 @@ __device__ __forceinline__ float exp2_hw(float y) {
 // (group 4, mean) gets its own instantiation: straight-line epilogues instead of uniform branches
 // and compute-both-then-select.
 template <typename T, bool LOGITS, int GPC, int RMAXC>
-__global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_OCC : 1)) void score_kernel(ScoreArgs p) {
+__global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_kernel(ScoreArgs p) {
   typedef Mma<T> M;
   const int GpV = GPC > 0 ? GPC : p.Gp;
   const int gsV = GPC == 8 ? 3 : GPC == 4 ? 2 : GPC == 2 ? 1 : p.gs;
@@ -232,9 +213,6 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
   vec16 pre[STAGE_IT];
 
   auto issue_loads = [&](int tile) {
-#ifdef ZP_DBG_NOLOAD
-    return;
-#endif
     const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
     const char* src = kbase + (int64_t)vpage[vp] * p.k_sp * T::bytes + (int64_t)toff * k_row;
 #pragma unroll
@@ -315,7 +293,7 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
       for (int r = 0; r < 16; ++r) run[r] = PASS == 0 ? -INFINITY : 0.f;
       // The middle sweep walks the tiles backwards: it starts on the tiles the first sweep read
       // last (still in L2) and ends on those the third sweep reads first.
-      auto order = [&](int i) { return (ZP_SCORE_ZIGZAG && PASS == 1) ? ntiles - 1 - i : i; };
+      auto order = [&](int i) { return PASS == 1 ? ntiles - 1 - i : i; };
       if (ntiles > 0) {
         issue_loads(order(0));
         commit_loads(kbuf0);
@@ -329,11 +307,7 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
         const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
         const int j = vslot[vp] & 0xffff;
         const bool last = (vslot[vp] >> 30) & 1;
-#ifdef ZP_DBG_NOCOMPUTE
-        if (false) {
-#else
         if (active) {
-#endif
 #pragma unroll 1
           for (int sti = 0; sti < NSUB; ++sti) {
             const int st = tg * NSUB + sti;
@@ -524,12 +498,9 @@ __global__ __launch_bounds__(kThreads, (kWaves == 4 && T::bytes == 2 ? ZP_SCORE_
         __syncthreads();
       }
     };
-#ifndef ZP_DBG_SWEEPS
-#define ZP_DBG_SWEEPS 7
-#endif
-    if (ZP_DBG_SWEEPS & 1) sweep(std::integral_constant<int, 0>{});
-    if (ZP_DBG_SWEEPS & 2) sweep(std::integral_constant<int, 1>{});
-    if (ZP_DBG_SWEEPS & 4) sweep(std::integral_constant<int, 2>{});
+    sweep(std::integral_constant<int, 0>{});
+    sweep(std::integral_constant<int, 1>{});
+    sweep(std::integral_constant<int, 2>{});
   }
 }
 
