@@ -52,21 +52,22 @@ def _check_properties(wl, flag, scores, k_before, v_before, shared_pages=()):
     # selector against the oracle on the GPU's own scores
     want = O.topk_mask(scores.cpu().view(L, B, Hkv, T), kk)
     assert torch.equal(f.cpu(), want)
-    # stable gather, checked densely on the device for layer 0
+    # stable gather, checked densely on the device, layer by layer
     enc = wl.block_tables
-    src_k = _gather_rows(k_before, enc, None)          # (B, T, Hkv, D) from the saved copy
-    src_v = _gather_rows(v_before, enc, None)
     tgt = wl.targets[:, :BUDGET].long()
-    got_k = wl.k[0][tgt.flatten()].view(B, kk, Hkv, -1)
-    got_v = wl.v[0][tgt.flatten()].view(B, kk, Hkv, -1)
-    for h in range(Hkv):
-        keep = f[0, :, h]                               # (B, T)
-        order = torch.argsort((~keep).to(torch.int8), dim=1, stable=True)[:, :kk]  # kept, ascending
-        idx = order.unsqueeze(-1).expand(B, kk, src_k.shape[-1])
-        assert torch.equal(got_k[:, :, h], torch.gather(src_k[:, :, h], 1, idx))
-        assert torch.equal(got_v[:, :, h], torch.gather(src_v[:, :, h], 1, idx))
+    for l in range(L):
+        src_k = _gather_rows(k_before, enc, None, l)     # (B, T, Hkv, D) from the saved copy
+        src_v = _gather_rows(v_before, enc, None, l)
+        got_k = wl.k[l][tgt.flatten()].view(B, kk, Hkv, -1)
+        got_v = wl.v[l][tgt.flatten()].view(B, kk, Hkv, -1)
+        for h in range(Hkv):
+            keep = f[l, :, h]                           # (B, T)
+            order = torch.argsort((~keep).to(torch.int8), dim=1, stable=True)[:, :kk]  # kept, ascending
+            idx = order.unsqueeze(-1).expand(B, kk, src_k.shape[-1])
+            assert torch.equal(got_k[:, :, h], torch.gather(src_k[:, :, h], 1, idx))
+            assert torch.equal(got_v[:, :, h], torch.gather(src_v[:, :, h], 1, idx))
     for p in shared_pages:
-        assert torch.equal(wl.k[0, p], k_before[0, p]) and torch.equal(wl.v[0, p], v_before[0, p])
+        assert torch.equal(wl.k[:, p], k_before[:, p]) and torch.equal(wl.v[:, p], v_before[:, p])
 
 
 def _save_touched(wl):
@@ -139,6 +140,24 @@ def test_config4_prefix_sharing_copy_on_write(dev):
     flag, scores = _run_pipeline(wl, cfg)
     _check_properties(wl, flag, scores, kb, vb, shared_pages=shared)
     _oracle_sample(wl, sub, kw, [0, 16, 255], scores, torch.bfloat16)
+
+
+def test_config4_layer_chunk_of_four(dev):
+    """The same 256-sequence shared-prefix batch as a chunk of four layers in one call (the
+    runner's `layer_stride` loop, zipage/engine/model_runner.py:466-469): the grid spans layers,
+    every layer has its own keys, queries and flags, and every layer's compaction is checked."""
+    from zipage_amd.compress import CompressConfig
+    from zipage_amd.workload import cpu_subset, ragged_batch
+    wl = ragged_batch(256, L=4, pool_pages=6000, budget=BUDGET, W=32, seed=3, lengths=(2049, 2560),
+                      shared_prefix_group=16, shared_prefix_pages=2)
+    shared = sorted({t[0] for t in wl.tables} | {t[1] for t in wl.tables})
+    kb, vb = _save_touched(wl)
+    sub = cpu_subset(wl, [7, 200])
+    kw = dict(enable_pooling=True, pooling_size=7)
+    flag, scores = _run_pipeline(wl, CompressConfig(budget_blocks=BUDGET, query_cache_len=32, **kw))
+    assert flag.shape[0] == 4 and not torch.equal(flag[0], flag[3])
+    _check_properties(wl, flag, scores, kb, vb, shared_pages=shared)
+    _oracle_sample(wl, sub, kw, [7, 200], scores, torch.bfloat16)
 
 
 def test_config1_single_sequence_fp32_full_oracle(dev):

@@ -36,6 +36,7 @@ constexpr int kRowWaves = 4;   // most waves along the query-row axis; the other
                                // Fewer row blocks (small window x group) use 2 or 1 row waves so
                                // that no wave idles: ScoreArgs::RW.
 constexpr int kDmax = 128;
+constexpr float kRefSpan = 60.f;   // exp(60) * 2^16 tokens stays far inside the fp32 range
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
@@ -267,8 +268,18 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
     float cl[16], mx[16];   // cl = -log2(row sum): p = 2^(x*log2(e) + cl)
 #pragma unroll
     for (int r = 0; r < 16; ++r) { mx[r] = 0.f; cl[r] = -INFINITY; }
+    // fp32 caches only (PASS 3): this lane's reference logit and running maximum per row
+    float ref[T::bytes == 4 ? 16 : 1], mrun[T::bytes == 4 ? 16 : 1];
+    bool far_off = false;   // PASS 3: a logit more than kRefSpan above its lane's reference
 
-    // One sweep over the sequence's K tiles.  PASS 0: row max; 1: row sum of exp; 2: output.
+    // One sweep over the sequence's K tiles.  PASS 0: row max; 1: row sum of exp; 2: output;
+    // 3 (fp32 caches): row max AND row sum in one sweep.  Without roundings to a 16-bit dtype the
+    // softmax does not depend on which finite reference is subtracted before the exponential, so
+    // every lane sums exp(s - ref) against its own first logit of the row, tracks its maximum,
+    // and the lanes' sums are brought to the common maximum afterwards:
+    // sum_t exp(s_t - m) = sum_lanes exp(ref_lane - m) sum_{t in lane} exp(s_t - ref_lane).
+    // Exact as long as no logit lies more than kRefSpan above its lane's reference (fp32 range);
+    // otherwise the caller falls back to the two separate sweeps.
     auto sweep = [&](auto pass_c) {
       constexpr int PASS = decltype(pass_c)::value;
       auto finish_tile = [&](int tile, int j, int toff) {
@@ -291,6 +302,10 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
       float run[16];
 #pragma unroll
       for (int r = 0; r < 16; ++r) run[r] = PASS == 0 ? -INFINITY : 0.f;
+      if constexpr (PASS == 3) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { mrun[r] = -INFINITY; ref[r] = 0.f; }
+      }
       // The middle sweep walks the tiles backwards: it starts on the tiles the first sweep read
       // last (still in L2) and ends on those the third sweep reads first.
       auto order = [&](int i) { return PASS == 1 ? ntiles - 1 - i : i; };
@@ -345,7 +360,16 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
                 if (slot > p.BS - p.W + w) acc[r] = -sgn * INFINITY;
               }
             }
-            if constexpr (PASS == 0) {
+            if constexpr (PASS == 3) {
+              const bool first = it == 0 && sti == 0;   // uniform
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                const float sv = acc[r] * p.scale;      // masked entries: -inf
+                if (first) ref[r] = sv > -INFINITY ? sv : 0.f;
+                mrun[r] = vmax(mrun[r], sv);
+                run[r] += exp2_hw((sv - ref[r]) * 1.44269504088896340736f);
+              }
+            } else if constexpr (PASS == 0) {
               // max of sign(scale)*acc; scaling is monotone, so it is applied once at the end
               if (sgn > 0.f) {  // block-uniform: the negation is a free source modifier
 #pragma unroll
@@ -470,7 +494,52 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
       }
       // the xor butterfly leaves the row result in all 32 lanes that share the row; the
       // token-group waves that share a row block then combine their halves through LDS
-      if constexpr (PASS < 2) {
+      if constexpr (PASS == 3) {
+        // row maximum over the 32 lanes of the row and the token-group waves, then the lanes' sums
+        // at that maximum
+        float mrow[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          far_off |= mrun[r] - ref[r] > kRefSpan;
+          const float v = half_max(mrun[r]);
+          mrow[r] = v;
+          if (col == 0) stat[wave * 32 + (r >> 2) * 8 + half * 4 + (r & 3)] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float v = mrow[r];
+#pragma unroll
+          for (int g2 = 1; g2 < TW; ++g2) {
+            const int ow = ((tg + g2) % TW) * RW + rbw;
+            v = fmaxf(v, stat[ow * 32 + (r >> 2) * 8 + half * 4 + (r & 3)]);
+          }
+          mx[r] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          // a lane that saw only masked tokens has run == 0 and contributes nothing
+          const float t = run[r] * exp2_hw((ref[r] - mx[r]) * 1.44269504088896340736f);
+          const float v = half_sum(run[r] > 0.f ? t : 0.f);
+          run[r] = v;
+          if (col == 0) stat[wave * 32 + (r >> 2) * 8 + half * 4 + (r & 3)] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          float v = run[r];
+#pragma unroll
+          for (int g2 = 1; g2 < TW; ++g2) {
+            const int ow = ((tg + g2) % TW) * RW + rbw;
+            v += stat[ow * 32 + (r >> 2) * 8 + half * 4 + (r & 3)];
+          }
+          const int m = row0 + (r >> 2) * 8 + (r & 3);
+          const bool ok = active && (m >> gsV) < p.W && (m & (GpV - 1)) < p.G;
+          cl[r] = ok ? -__builtin_amdgcn_logf(v) : -INFINITY;
+        }
+        __syncthreads();
+      } else if constexpr (PASS < 2) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const float v = PASS == 0 ? half_max(run[r]) : half_sum(run[r]);
@@ -498,8 +567,15 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
         __syncthreads();
       }
     };
-    sweep(std::integral_constant<int, 0>{});
-    sweep(std::integral_constant<int, 1>{});
+    bool merged = false;
+    if constexpr (T::bytes == 4 && !LOGITS) {
+      sweep(std::integral_constant<int, 3>{});
+      merged = !__syncthreads_or(far_off ? 1 : 0);
+    }
+    if (!merged) {
+      sweep(std::integral_constant<int, 0>{});
+      sweep(std::integral_constant<int, 1>{});
+    }
     sweep(std::integral_constant<int, 2>{});
   }
 }
