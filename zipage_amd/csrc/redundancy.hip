@@ -343,8 +343,8 @@ __global__ __launch_bounds__(NW * 64) void gram_kernel(GramArgs p) {
 // ------------------------------------------------------------------ fp32 caches, lightning, whole page in LDS
 // One workgroup per (layer, sequence, head, page) of at most 256 keys: the page is loaded once
 // with coalesced 16-byte loads, normalised on the way into LDS (132 KB), and after ONE barrier
-// every wave multiplies its 32 rows (A operand read from the same LDS copy) with all column
-// blocks: no tile pipeline, no further barriers, no strided per-lane row loads.
+// every wave multiplies its 32 rows (A operand read from the same LDS copy) with its share of the
+// column blocks (every unordered pair of blocks once): no tile pipeline, no strided row loads.
 constexpr int kPage32Rows = 256;
 constexpr int kPage32Threads = 512;
 __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs p) {
@@ -355,9 +355,9 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
   extern __shared__ __align__(16) char smem[];
   float* kpl = (float*)smem;                                   // [256][ROWF] normalised keys
   unsigned long long* l_corr = (unsigned long long*)(kpl + kPage32Rows * ROWF);
-  float* l_sum = (float*)(l_corr + kPage32Rows);
-  float* l_val = l_sum + kPage32Rows;
-  int* l_col = (int*)(l_val + kPage32Rows);
+  unsigned long long* l_claim = l_corr + kPage32Rows;       // (claimed index + 1) << 32 | value bits
+  float* l_sum = (float*)(l_claim + kPage32Rows);
+  float* l_csum = l_sum + kPage32Rows;                        // [4][256] column sums per distance
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
@@ -389,7 +389,7 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
       raw[it] = *(const float4*)(page + (int64_t)(row < p.BS ? row : 0) * k_row +
                                  (piece < dpieces ? piece : 0) * 16);
     }
-    if (tid < kPage32Rows) l_corr[tid] = 0ull;
+    if (tid < kPage32Rows) { l_corr[tid] = 0ull; l_claim[tid] = 0ull; }
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int row = it * ROWS_PER_IT + row0;
@@ -403,6 +403,13 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
   }
   __syncthreads();
 
+  // ---- Gram tiles, every unordered pair of 32-key blocks once: wave a multiplies its block with
+  // the blocks (a + d) mod n, d = 0 .. n/2 (the last distance only for the lower half of the
+  // waves when n is even).  A tile off the diagonal block serves both of its sides: the rows get
+  // their partial row sums and claims as before, the columns get the tile's column sums
+  // (slot [d][key], written by exactly one wave, added in a fixed order at the end) and the last
+  // ROW over the threshold as their claim.  Claims travel as (index, value) pairs through one
+  // 64-bit atomicMax per key, so the result does not depend on the order of the waves.
   const int nrb = p.BS / 32;
   if (wave < nrb) {
     const int rb = wave;
@@ -420,8 +427,10 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
     int ccol[16];
 #pragma unroll
     for (int r = 0; r < 16; ++r) { rsum[r] = 0.f; cval[r] = 0.f; ccol[r] = -1; }
+    const int nd = nrb / 2 + (((nrb & 1) || rb < nrb / 2) ? 1 : 0);   // distances 0 .. nd-1
 #pragma unroll 1
-    for (int cb = 0; cb < nrb; ++cb) {
+    for (int d = 0; d < nd; ++d) {
+      const int cb = rb + d < nrb ? rb + d : rb + d - nrb;
       f32x16_t acc;
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[r] = 0.f;
@@ -435,13 +444,27 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
         acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 3], bv.w, acc, 0, 0, 0);
       }
       const int cslot = cb * 32 + col;
+      float csum = 0.f, rv = 0.f;     // column side: sum over this lane's rows, last row over the threshold
+      int rlast = -1;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
         float sv = acc[r];
         if (rslot == cslot) sv = 0.f;
         rsum[r] += sv;
-        if (sv > p.threshold) { ccol[r] = cslot; cval[r] = sv; }
+        csum += sv;
+        const bool over = sv > p.threshold;
+        if (over && cslot > ccol[r]) { ccol[r] = cslot; cval[r] = sv; }
+        if (over) { rlast = rslot; rv = sv; }     // rslot grows with r inside a lane
+      }
+      if (d != 0) {
+        csum += lane_xor32(csum);
+        if (half == 0) l_csum[(d - 1) * kPage32Rows + cslot] = csum;
+        const int orl = lane_xor32(rlast);
+        const float orv = lane_xor32(rv);
+        if (orl > rlast) { rlast = orl; rv = orv; }
+        if (half == 0 && rlast >= 0)
+          atomicMax(&l_claim[cslot], ((unsigned long long)(unsigned)(rlast + 1) << 32) | __float_as_uint(rv));
       }
     }
 #pragma unroll
@@ -453,19 +476,31 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
       if (col == 0) {
         const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
         l_sum[rslot] = sv;
-        l_col[rslot] = c;
-        l_val[rslot] = v;
+        if (c >= 0)
+          atomicMax(&l_claim[rslot], ((unsigned long long)(unsigned)(c + 1) << 32) | __float_as_uint(v));
       }
     }
   }
   __syncthreads();
   for (int j = tid; j < p.BS; j += kPage32Threads) {
-    const int c = l_col[j];
-    if (c >= 0 && c < p.BS) atomicAdd(&l_corr[c], to_fixed32(l_val[j]));
+    const unsigned long long cl = l_claim[j];
+    const int c = (int)(cl >> 32) - 1;
+    if (c >= 0 && c < p.BS) atomicAdd(&l_corr[c], to_fixed32(__uint_as_float((unsigned)cl)));
   }
   __syncthreads();
-  for (int i = tid; i < p.BS; i += kPage32Threads)
-    Elem<T>::st(p.r_out, obase + i, l_sum[i] - from_fixed32(l_corr[i]));
+  const int ndist = nrb / 2;     // column-side slots in use: distances 1 .. nrb/2
+  for (int i = tid; i < p.BS; i += kPage32Threads) {
+    float sv = l_sum[i];
+    const int blk = i >> 5;
+    for (int d = 1; d <= ndist; ++d) {
+      // the wave that wrote slot [d][i] is block (blk - d) mod n; with n even the last distance
+      // is only run by the lower half of the waves
+      const int a = blk - d >= 0 ? blk - d : blk - d + nrb;
+      const bool ran = d < nrb / 2 + (((nrb & 1) || a < nrb / 2) ? 1 : 0);
+      if (ran) sv += l_csum[(d - 1) * kPage32Rows + i];
+    }
+    Elem<T>::st(p.r_out, obase + i, sv - from_fixed32(l_corr[i]));
+  }
 }
 
 // ------------------------------------------------------------------ 16-bit caches: split-bf16 Gram
@@ -1630,7 +1665,7 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
   }
   if constexpr (T::bytes == 4 && !RAW) {
     if (a.BS <= kPage32Rows && a.BS % 32 == 0) {
-      const size_t smem = (size_t)kPage32Rows * ROWF * 4 + (size_t)kPage32Rows * 20;
+      const size_t smem = (size_t)kPage32Rows * ROWF * 4 + (size_t)kPage32Rows * (8 + 8 + 4 + 4 * 4);
       if (hipFuncSetAttribute((const void*)gram_page_f32_kernel,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
         zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
