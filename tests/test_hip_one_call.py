@@ -79,3 +79,36 @@ def test_one_call_rejects_a_short_workspace(dev):
         _lib.call("zp_compress_layers", k.data_ptr(), v.data_ptr(), q.data_ptr(), 0, qid.data_ptr(),
                   enc.data_ptr(), comp.data_ptr(), target.data_ptr(), 0, *dims, strides, 0,
                   ctypes.byref(cc), ws.data_ptr(), need - 256, None, 0)
+
+
+@pytest.mark.parametrize("kw", [dict(enable_pooling=True, pooling_size=5),
+                                dict(use_global_score=True, decay_factor=0.8)],
+                         ids=["pooling", "global-score"])
+def test_one_call_on_rows_too_long_for_the_one_launch_selection(dev, kw):
+    """A sequence of 80 pages (20 480 tokens) does not fit the one-launch selection's LDS row:
+    zp_compress_layers then runs pooling, the mask epilogue and top-k as separate launches on
+    copies inside its workspace (the carried scores still come from the untouched scores).  Same
+    bits as the separate entry points called from Python."""
+    from zipage_amd.compress import CompressConfig, StageTimer, _compress_layers_one_call, compress_layers
+    from oracle.zipage_oracle import encode_block_table
+    dtype, L, Hkv, Hq, W, budget, NB = torch.bfloat16, 1, 1, 2, 16, 8, 80
+    tables = [list(range(NB)), list(range(NB, NB + 12))]
+    enc = encode_block_table(tables)
+    target = torch.tensor([t[:budget + 1] for t in tables], dtype=torch.int32)
+    k, v, q, sc = cases.make_caches(5, L, NB + 12, 256, Hkv, Hq, 128, W, 2, dtype, with_score_cache=True)
+    qid = torch.arange(2, dtype=torch.int32)
+    comp = torch.tensor([True, False])
+    cfg = CompressConfig(budget_blocks=budget, query_cache_len=W, **kw)
+    outs = []
+    for one_call in (True, False):
+        gk, gv, gsc = k.clone().to(dev), v.clone().to(dev), sc.clone().to(dev)
+        args = (gk, gv, q.to(dev), gsc, qid.to(dev), enc.to(dev), comp.to(dev), target.to(dev), cfg)
+        if one_call:
+            flag = _compress_layers_one_call(*args, StageTimer(False), True)
+        else:
+            flag = compress_layers(*args, fused_select=False)
+        torch.cuda.synchronize()
+        outs.append((flag.cpu(), gk.cpu(), gv.cpu(), gsc.cpu()))
+    for a, b in zip(*outs):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+    assert (outs[0][0].flatten(3).sum(-1) == budget * 256).all()
