@@ -152,6 +152,18 @@ __device__ __forceinline__ int wave_sum_i(int v) {
   v += lane_xor16(v);
   return v + lane_xor32(v);
 }
+// Inclusive prefix sum over the 64 lanes of a wave in six DPP adds: shifts by 1, 2, 4 and 8 inside
+// each row of 16 lanes (lanes without a source add 0), then lane 15 of rows 0 / 2 is added to rows
+// 1 / 3 and lane 31 to the upper half.
+__device__ __forceinline__ int wave_prefix_sum_incl(int v) {
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, false);   // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, false);   // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, false);   // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, false);   // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);   // row_bcast:15 -> rows 1, 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);   // row_bcast:31 -> rows 2, 3
+  return v;
+}
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 __device__ __forceinline__ int wave_id() { return threadIdx.x >> 6; }
 __device__ __forceinline__ uint64_t lanemask_lt() {

@@ -49,9 +49,9 @@ __global__ __launch_bounds__(kThreads) void pool_kernel(
     const void* __restrict__ in, void* __restrict__ out, const uint8_t* __restrict__ compressed,
     int B, int Hkv, int Tn, int ksize, int continues, int mode) {
   extern __shared__ float row[];
-  const int64_t r = blockIdx.x;
-  const int b = (int)((r / Hkv) % B);
-  const int64_t base = r * Tn;
+  const uint32_t r = blockIdx.x;          // 32-bit: a 64-bit division costs hundreds of scalar instructions
+  const int b = (int)((r / (uint32_t)Hkv) % (uint32_t)B);
+  const int64_t base = (int64_t)r * Tn;
   const bool raw = !continues && compressed[b] != 0;
   if (raw) {
     for (int t = threadIdx.x; t < Tn; t += kThreads)
@@ -94,10 +94,10 @@ __global__ __launch_bounds__(kThreads) void epilogue_kernel(
     int B, int NB, int BS, int Hkv, int norm_s, int norm_r, float lam, float one_minus_lam,
     int sink_len, int window, int mask_pad) {
   __shared__ float red_lds[kThreads / 64];
-  const int64_t r = blockIdx.x;
-  const int b = (int)((r / Hkv) % B);
+  const uint32_t r = blockIdx.x;          // 32-bit: a 64-bit division costs hundreds of scalar instructions
+  const int b = (int)((r / (uint32_t)Hkv) % (uint32_t)B);
   const int Tn = NB * BS;
-  const int64_t base = r * Tn;
+  const int64_t base = (int64_t)r * Tn;
   const int32_t* trow = table + (int64_t)b * NB;
   float smax = 1.f, rmax = 1.f;
   if (norm_s) {
