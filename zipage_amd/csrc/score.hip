@@ -172,7 +172,21 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
 
   // ---- valid page list (block-uniform), zero pad-page outputs
   __shared__ int nvalid_s;
-  if (tid == 0) {
+  if (p.NB <= 64) {
+    // one lane per table entry; a ballot packs the usable pages in table order
+    if (wave == 0) {
+      const int code = lane < p.NB ? p.table[(int64_t)b * p.NB + lane] : -1;
+      const int pid = page_is_pad(code) ? -1 : page_id(code);
+      const bool ok = pid >= 0 && pid < p.num_pages;
+      const unsigned long long okm = __builtin_amdgcn_ballot_w64(ok);
+      if (ok) {
+        const int n = __builtin_popcountll(okm & lanemask_lt());
+        vpage[n] = pid;
+        vslot[n] = lane | (page_is_last(code) ? (1 << 30) : 0);
+      }
+      if (lane == 0) nvalid_s = __builtin_popcountll(okm);
+    }
+  } else if (tid == 0) {
     int n = 0;
     for (int j = 0; j < p.NB; ++j) {
       const int code = p.table[(int64_t)b * p.NB + j];
@@ -185,8 +199,9 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
     }
     nvalid_s = n;
   }
-  // LDS tiles start zeroed so that head_dim < 128 contributes nothing
-  for (int i = tid; i < 2 * TN * ROWB / 4; i += kThreads) ((uint32_t*)smem)[i] = 0u;
+  // with a head dim below 128 the tail of every LDS row must read as zero
+  if (p.D * T::bytes < kDmax * T::bytes)
+    for (int i = tid; i < 2 * TN * ROWB / 4; i += kThreads) ((uint32_t*)smem)[i] = 0u;
   __syncthreads();
   const int nvalid = nvalid_s;
   {
@@ -205,22 +220,29 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
 
   const int tiles_per_page = p.BS / TN;
   const int ntiles = nvalid * tiles_per_page;
+  // tile -> (valid page, token offset); a shift when a page holds a power-of-two number of tiles
+  const int tpp_shift = (tiles_per_page & (tiles_per_page - 1)) == 0 ? __builtin_ctz(tiles_per_page) : -1;
+  auto tile_page = [&](int tile) { return tpp_shift >= 0 ? tile >> tpp_shift : tile / tiles_per_page; };
   const int dpieces = p.D * T::bytes / 16;  // valid 16-byte pieces per key row
   const int64_t k_row = (int64_t)p.Hkv * p.D * T::bytes;
   const char* kbase = p.k + (l * p.k_sl) * T::bytes + (int64_t)h * p.D * T::bytes;
 
-  // staging coordinates of this thread
+  // staging coordinates of this thread; the byte offsets of its eight pieces inside a tile are
+  // kept as 32-bit registers and the tile base is wave-uniform, so a load needs no address math
   const int st_piece = tid % PIECES, st_row0 = tid / PIECES;
   vec16 pre[STAGE_IT];
+  uint32_t ld_off[STAGE_IT];
+#pragma unroll
+  for (int i = 0; i < STAGE_IT; ++i)
+    ld_off[i] = (uint32_t)((st_row0 + i * ROWS_PER_IT) * k_row + st_piece * 16);
 
   auto issue_loads = [&](int tile) {
-    const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
-    const char* src = kbase + (int64_t)vpage[vp] * p.k_sp * T::bytes + (int64_t)toff * k_row;
+    const int vp = tile_page(tile), toff = (tile - vp * tiles_per_page) * TN;
+    const int pid = __builtin_amdgcn_readfirstlane(vpage[vp]);
+    const char* src = kbase + (int64_t)pid * p.k_sp * T::bytes + (int64_t)toff * k_row;
 #pragma unroll
     for (int i = 0; i < STAGE_IT; ++i) {
-      const int row = st_row0 + i * ROWS_PER_IT;
-      if (st_piece < dpieces)
-        pre[i] = *(const vec16*)(src + (int64_t)row * k_row + st_piece * 16);
+      if (st_piece < dpieces) pre[i] = *(const vec16*)(src + ld_off[i]);
     }
   };
   auto commit_loads = [&](char* buf) {
@@ -319,12 +341,59 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
         char* cur = (it & 1) ? kbuf1 : kbuf0;
         char* nxt = (it & 1) ? kbuf0 : kbuf1;
         if (it + 1 < ntiles) issue_loads(order(it + 1));
-        const int vp = tile / tiles_per_page, toff = (tile - vp * tiles_per_page) * TN;
-        const int j = vslot[vp] & 0xffff;
-        const bool last = (vslot[vp] >> 30) & 1;
+        const int vp = tile_page(tile), toff = (tile - vp * tiles_per_page) * TN;
+        const int vs = __builtin_amdgcn_readfirstlane(vslot[vp]);
+        const int j = vs & 0xffff;
+        const bool last = (vs >> 30) & 1;
         if (active) {
+          int sti = 0;
+          if constexpr (PASS == 0 && !LOGITS && T::bytes == 2) {
+            // The max sweep has little to do per product, so a lone chain of eight dependent MFMAs
+            // behind an LDS round trip leaves the matrix core idle half of the time: two subtiles
+            // are multiplied at once, their MFMAs alternating between two accumulators.
 #pragma unroll 1
-          for (int sti = 0; sti < NSUB; ++sti) {
+            for (; sti + 1 < NSUB; sti += 2) {
+              const int st = tg * NSUB + sti;
+              const char* browA = cur + (st * 32 + col) * ROWB + half * M::EPL * T::bytes;
+              const char* browB = browA + 32 * ROWB;
+              f32x16_t accA, accB;
+#pragma unroll
+              for (int r = 0; r < 16; ++r) { accA[r] = 0.f; accB[r] = 0.f; }
+              constexpr int KH = KS / 2;
+#pragma unroll
+              for (int s0 = 0; s0 < KS; s0 += KH) {
+                Frag bA[KH], bB[KH];
+#pragma unroll
+                for (int s = 0; s < KH; ++s) bA[s] = *(const Frag*)(browA + (s0 + s) * M::KPI * T::bytes);
+#pragma unroll
+                for (int s = 0; s < KH; ++s) bB[s] = *(const Frag*)(browB + (s0 + s) * M::KPI * T::bytes);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int s = 0; s < KH; ++s) {
+                  accA = M::mma(afrag[s0 + s], bA[s], accA);
+                  accB = M::mma(afrag[s0 + s], bB[s], accB);
+                }
+              }
+              if (last && (toff + st * 32 + 63 > p.BS - p.W)) {
+                const int slotA = toff + st * 32 + col;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                  const int w = (row0 + (r >> 2) * 8 + (r & 3)) >> gsV;
+                  if (slotA > p.BS - p.W + w) accA[r] = -sgn * INFINITY;
+                  if (slotA + 32 > p.BS - p.W + w) accB[r] = -sgn * INFINITY;
+                }
+              }
+              if (sgn > 0.f) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) run[r] = vmax(vmax(run[r], accA[r]), accB[r]);
+              } else {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) run[r] = vmax_neg(vmax_neg(run[r], accA[r]), accB[r]);
+              }
+            }
+          }
+#pragma unroll 1
+          for (; sti < NSUB; ++sti) {
             const int st = tg * NSUB + sti;
             f32x16_t acc;
 #pragma unroll
