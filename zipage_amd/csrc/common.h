@@ -99,7 +99,12 @@ __device__ __forceinline__ int page_id(int code) { return code < -1 ? -code - 2 
 // gfx950 lane-swap instructions for the two wider steps.  A ds_bpermute round trip costs a
 // hundred-odd cycles of latency; these are ordinary VALU instructions.
 template <int N> __device__ __forceinline__ int dpp_row_ror(int x) {
-  return __builtin_amdgcn_update_dpp(0, x, 0x120 + N, 0xf, 0xf, false);  // lane i <- lane (i+N)%16 of its row
+  return __builtin_amdgcn_update_dpp(0, x, 0x120 + N, 0xf, 0xf, false);  // lane i <- lane (i-N)%16 of its row
+}
+// lane i <- lane i+N of its row of 16 (0 where that lane lies outside the row)
+template <int N> __device__ __forceinline__ float dpp_row_shl(float x) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x100 + N, 0xf, 0xf, false));
 }
 template <int N> __device__ __forceinline__ float dpp_row_ror(float x) {
   return __builtin_bit_cast(float, dpp_row_ror<N>(__builtin_bit_cast(int, x)));

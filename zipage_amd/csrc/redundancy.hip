@@ -798,6 +798,25 @@ template <> struct Mfma16<F16> {
   }
 };
 
+// A float as three 16-bit pieces of the cache dtype (hi + mid + lo carries its fp32 mantissa).
+template <typename T> struct Split3;
+template <> struct Split3<BF16> {
+  __device__ static __forceinline__ void run(float v, uint16_t* o) {
+    const float h = bf16_round(v), m = bf16_round(v - h), l = bf16_round(v - h - m);
+    o[0] = (uint16_t)(__float_as_uint(h) >> 16);
+    o[1] = (uint16_t)(__float_as_uint(m) >> 16);
+    o[2] = (uint16_t)(__float_as_uint(l) >> 16);
+  }
+};
+template <> struct Split3<F16> {
+  __device__ static __forceinline__ void run(float v, uint16_t* o) {
+    o[0] = float_to_f16_bits(v);
+    const float r1 = v - f16_bits_to_float(o[0]);
+    o[1] = float_to_f16_bits(r1);
+    o[2] = float_to_f16_bits(r1 - f16_bits_to_float(o[1]));
+  }
+};
+
 // The cosine matrix factors as S_ij = rn_i rn_j (k_i . k_j) with rn = 1 / norm: the raw 16-bit
 // keys go to the matrix cores as they are (one MFMA per k-step, exact products, fp32 sums) and
 // the two scale factors are applied to the accumulators.  One plane of raw keys in LDS (68 KB),
@@ -808,7 +827,7 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
   typedef typename Mfma16<T>::V frag_t;
   constexpr int PIECES = kDmax / 8;
   constexpr int KSB = kDmax / 16;
-  constexpr int PLANE = kPageRows * ROWH;
+  constexpr int PLANE = (kPageRows + 4) * ROWH;   // the page, then the three planes of the key sum
 
   extern __shared__ __align__(16) char smem[];
   char* k_pl = smem;                                                          // raw keys
@@ -839,42 +858,69 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
   const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
   const char* page = p.k + (l * p.k_sl + (int64_t)rpid * p.k_sp) * 2 + (int64_t)h * p.D * 2;
 
-  // ---- stage: copy the page, norms, sum of the normalised keys, row sums
-  {
-    const int piece = tid % PIECES, row0 = tid / PIECES;       // 32 rows per iteration
-    constexpr int ROWS_PER_IT = kPageThreads / PIECES;
-    constexpr int ITERS = kPageRows / ROWS_PER_IT;
-    // all loads of the page are in flight before the first one is consumed
-    u32x4 raw[ITERS];
-    float rn[ITERS], sq[ITERS];
+  // ---- copy the page into LDS; the raw keys also stay in registers for the key sum
+  const int piece = tid % PIECES, row0 = tid / PIECES;       // 32 rows per iteration
+  constexpr int ROWS_PER_IT = kPageThreads / PIECES;
+  constexpr int ITERS = kPageRows / ROWS_PER_IT;
+  u32x4 raw[ITERS];
 #pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-      const int row = it * ROWS_PER_IT + row0;
-      raw[it] = *(const u32x4*)(page + (int64_t)(row < p.BS ? row : 0) * k_row +
-                                (piece < dpieces ? piece : 0) * 16);
+  for (int it = 0; it < ITERS; ++it) {
+    const int row = it * ROWS_PER_IT + row0;
+    raw[it] = *(const u32x4*)(page + (int64_t)(row < p.BS ? row : 0) * k_row +
+                              (piece < dpieces ? piece : 0) * 16);
+  }
+  if (tid < kPageRows) { l_col[tid] = -1; l_corr[tid] = 0ull; }
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int row = it * ROWS_PER_IT + row0;
+    if (!(row < p.BS && piece < dpieces)) raw[it] = u32x4{0u, 0u, 0u, 0u};   // past the page / head dim: zeros
+    if (row < p.BS) *(u32x4*)(k_pl + row * ROWH + piece * 16) = raw[it];
+  }
+  __syncthreads();
+
+  // ---- norms from the diagonal of the Gram matrix: wave a multiplies its own block (a, a), which
+  // the claim rule needs anyway, and the 32 lanes that hold a diagonal entry turn it into 1 / norm
+  const int nrb = p.BS / 32;
+  const int a = wave;
+  frag_t ak[KSB];
+  f32x16_t diag;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) diag[r] = 0.f;
+  if (wave < nrb) {
+    const char* arow = k_pl + (a * 32 + col) * ROWH + half * 16;
+#pragma unroll
+    for (int s = 0; s < KSB; ++s) ak[s] = *(const frag_t*)(arow + s * 32);
+#pragma unroll
+    for (int s = 0; s < KSB; ++s) diag = Mfma16<T>::run(ak[s], ak[s], diag);
+    // lane (col, half) owns rows (r/4)*8 + half*4 + r%4 of column col: entry (col, col) is its
+    // register (col/8)*4 + col%4 when (col%8)/4 == half
+    const int my_r = (col >> 3) * 4 + (col & 3);
+    float ss = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) ss = r == my_r ? diag[r] : ss;
+    // the quotient only scales fp32 sums: the 1-ulp reciprocal is exact enough
+    const float rn = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr));
+    if (((col & 7) >> 2) == half) {
+      l_rn[a * 32 + col] = rn;
+      l_sum[a * 32 + col] = ss * rn * rn;      // |e_i|^2, taken off the row sum below
     }
-    if (tid < kPageRows) { l_col[tid] = -1; l_corr[tid] = 0ull; }
+  }
+  __syncthreads();
+
+  // ---- summed normalised key S = sum_j rn_j k_j (fp32, fixed order over the waves), stored as
+  // three 16-bit planes behind the page so that the matrix cores can multiply the keys with it
+  {
     float cs[8];
 #pragma unroll
     for (int q = 0; q < 8; ++q) cs[q] = 0.f;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
       const int row = it * ROWS_PER_IT + row0;
-      const bool ok = row < p.BS && piece < dpieces;
-      if (!ok) raw[it] = u32x4{0u, 0u, 0u, 0u};     // lanes past the page or the head dim hold zeros
-      if (row < p.BS) *(u32x4*)(k_pl + row * ROWH + piece * 16) = raw[it];
+      const float rn = row < p.BS ? l_rn[row] : 0.f;
       float e[8];
       Unpack<T>::run(vec16{raw[it].x, raw[it].y, raw[it].z, raw[it].w}, e);
-      float ss = 0.f;
 #pragma unroll
-      for (int q = 0; q < 8; ++q) ss = fmaf(e[q], e[q], ss);
-      ss = pieces_sum<PIECES>(ss);
-      // the quotient only scales fp32 sums: the 1-ulp reciprocal is exact enough
-      rn[it] = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr));
-      sq[it] = ss * rn[it] * rn[it];
-      if (piece == 0 && row < p.BS) l_rn[row] = rn[it];
-#pragma unroll
-      for (int q = 0; q < 8; ++q) cs[q] = fmaf(e[q], rn[it], cs[q]);
+      for (int q = 0; q < 8; ++q) cs[q] = fmaf(e[q], rn, cs[q]);
     }
     // the four key rows a wave handles per iteration sit 16 lanes apart
 #pragma unroll
@@ -887,44 +933,46 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
       *(float4*)dst = make_float4(cs[0], cs[1], cs[2], cs[3]);
       *(float4*)(dst + 4) = make_float4(cs[4], cs[5], cs[6], cs[7]);
     }
-    __syncthreads();
-    // summed key (fixed order over the waves), then every key's dot product with the rest:
-    // e_i . (S - e_i) = rn_i (k_i . S) - |e_i|^2
-    float sv[8];
-#pragma unroll
-    for (int q = 0; q < 8; ++q) sv[q] = 0.f;
-#pragma unroll
-    for (int w = 0; w < kPageWaves; ++w) {
-      const float* src = l_part + w * kDmax + piece * 8;
-      const float4 a = *(const float4*)src, c = *(const float4*)(src + 4);
-      sv[0] += a.x; sv[1] += a.y; sv[2] += a.z; sv[3] += a.w;
-      sv[4] += c.x; sv[5] += c.y; sv[6] += c.z; sv[7] += c.w;
-    }
-#pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-      const int row = it * ROWS_PER_IT + row0;
-      float e[8];
-      Unpack<T>::run(vec16{raw[it].x, raw[it].y, raw[it].z, raw[it].w}, e);
-      float t = 0.f;
-#pragma unroll
-      for (int q = 0; q < 8; ++q) t = fmaf(e[q], sv[q], t);
-      t = pieces_sum<PIECES>(t);
-      if (piece == 0 && row < p.BS) l_sum[row] = t * rn[it] - sq[it];
-    }
   }
+  __syncthreads();
+  if (tid < kDmax) {
+    float sv = 0.f;
+#pragma unroll
+    for (int w = 0; w < kPageWaves; ++w) sv += l_part[w * kDmax + tid];
+    uint16_t o[3];
+    Split3<T>::run(sv, o);
+#pragma unroll
+    for (int pl = 0; pl < 3; ++pl) *(uint16_t*)(k_pl + (kPageRows + pl) * ROWH + tid * 2) = o[pl];
+  }
+  __syncthreads();
 
   // ---- Gram tiles: wave a owns row block a and the column blocks (a + d) mod n
-  const int nrb = p.BS / 32;
   if (wave < nrb) {
-    const int a = wave;
-    frag_t ak[KSB];
     float rn_row[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) rn_row[r] = l_rn[a * 32 + (r >> 2) * 8 + half * 4 + (r & 3)];
+    // row sums without the matrix: sum_{j != i} e_i.e_j = rn_i (k_i . S) - |e_i|^2, the products
+    // k_i . S as one more tile whose columns 0..2 are the planes of S
     {
-      const char* arow = k_pl + (a * 32 + col) * ROWH + half * 16;
+      f32x16_t acc;
 #pragma unroll
-      for (int s = 0; s < KSB; ++s) ak[s] = *(const frag_t*)(arow + s * 32);
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+      const char* srow = k_pl + (kPageRows + (col < 3 ? col : 0)) * ROWH + half * 16;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) rn_row[r] = l_rn[a * 32 + (r >> 2) * 8 + half * 4 + (r & 3)];
+      for (int s = 0; s < KSB; ++s) {
+        frag_t bk = *(const frag_t*)(srow + s * 32);
+        if (col >= 3) __builtin_memset(&bk, 0, sizeof(bk));
+        acc = Mfma16<T>::run(ak[s], bk, acc);
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        // lane col 0 adds the lo, mid and hi products (lanes col 2, 1, 0), smallest first
+        const float t = (dpp_row_shl<2>(acc[r]) + dpp_row_shl<1>(acc[r])) + acc[r];
+        if (col == 0) {
+          const int row = a * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+          l_sum[row] = t * rn_row[r] - l_sum[row];
+        }
+      }
     }
     // a tile whose largest entry stays below this cannot hold a claim (slack for the rounding of
     // the two ways the scale factors are multiplied in)
@@ -937,23 +985,22 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
     for (int d = 0; d < nd; ++d) {
       const int cb = a + d < nrb ? a + d : a + d - nrb;
       f32x16_t acc;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
       const char* brow = k_pl + (cb * 32 + col) * ROWH + half * 16;
       const int cslot = cb * 32 + col;
       const float rn_col = l_rn[cslot];
-      {
+      if (d == 0) {
+        // the diagonal block was multiplied for the norms; a key against itself counts as 0
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          acc[r] = (r >> 2) * 8 + half * 4 + (r & 3) == col ? 0.f : diag[r];
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
         frag_t bk[KSB];
 #pragma unroll
         for (int s = 0; s < KSB; ++s) bk[s] = *(const frag_t*)(brow + s * 32);
 #pragma unroll
         for (int s = 0; s < KSB; ++s) acc = Mfma16<T>::run(ak[s], bk[s], acc);
-      }
-      if (d == 0) {
-        // the diagonal block: a key against itself counts as 0
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-          if ((r >> 2) * 8 + half * 4 + (r & 3) == col) acc[r] = 0.f;
       }
       // most tiles hold no entry over the threshold: one maximum decides
       float big = -INFINITY;
@@ -1371,23 +1418,6 @@ __global__ __launch_bounds__(kThreads) void raw_claim_value_kernel(GramArgs p) {
 // a page's 256 keys with 32 chunks at a time run on the matrix cores: the keys as stored (exact
 // 16-bit products), s_chunk split into three 16-bit planes (together its full fp32 mantissa).
 // One workgroup per valid page; wave w owns keys 32 w .. 32 w + 31.
-template <typename T> struct Split3;
-template <> struct Split3<BF16> {
-  __device__ static __forceinline__ void run(float v, uint16_t* o) {
-    const float h = bf16_round(v), m = bf16_round(v - h), l = bf16_round(v - h - m);
-    o[0] = (uint16_t)(__float_as_uint(h) >> 16);
-    o[1] = (uint16_t)(__float_as_uint(m) >> 16);
-    o[2] = (uint16_t)(__float_as_uint(l) >> 16);
-  }
-};
-template <> struct Split3<F16> {
-  __device__ static __forceinline__ void run(float v, uint16_t* o) {
-    o[0] = float_to_f16_bits(v);
-    const float r1 = v - f16_bits_to_float(o[0]);
-    o[1] = float_to_f16_bits(r1);
-    o[2] = float_to_f16_bits(r1 - f16_bits_to_float(o[1]));
-  }
-};
 // chunk sums are below 16 + 1 in magnitude: 2^-26 fixed point fits 32 bits, and integer atomics
 // make the sum of several claims independent of their order
 __device__ __forceinline__ int to_fixed26(float v) { return (int)(v * 67108864.f); }
@@ -1651,7 +1681,7 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
   const size_t tail = (RAW ? 0 : (size_t)a.BS * 20) + sizeof(int) * 2 * a.NB;
   if constexpr (T::bytes == 2 && !RAW) {
     if (a.BS <= kPageRows && a.BS % 32 == 0) {
-      const size_t smem = (size_t)kPageRows * ROWH + (size_t)kPageRows * 20 +
+      const size_t smem = (size_t)(kPageRows + 4) * ROWH + (size_t)kPageRows * 20 +
                           (size_t)kPageWaves * kDmax * 4;
       if (hipFuncSetAttribute((const void*)gram_page_kernel<T>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
