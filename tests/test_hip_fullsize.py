@@ -50,8 +50,9 @@ def _check_properties(wl, flag, scores, k_before, v_before, shared_pages=()):
     win[..., BS - wl.W:] = True
     assert flag[last & win].all(), "the window slots of the last page are always kept"
     # selector against the oracle on the GPU's own scores
-    want = O.topk_mask(scores.cpu().view(L, B, Hkv, T), kk)
-    assert torch.equal(f.cpu(), want)
+    if scores is not None:
+        want = O.topk_mask(scores.cpu().view(L, B, Hkv, T), kk)
+        assert torch.equal(f.cpu(), want)
     # stable gather, checked densely on the device, layer by layer
     enc = wl.block_tables
     tgt = wl.targets[:, :BUDGET].long()
@@ -158,6 +159,44 @@ def test_config4_layer_chunk_of_four(dev):
     assert flag.shape[0] == 4 and not torch.equal(flag[0], flag[3])
     _check_properties(wl, flag, scores, kb, vb, shared_pages=shared)
     _oracle_sample(wl, sub, kw, [7, 200], scores, torch.bfloat16)
+
+
+def test_config4_36_layers_in_chunks_of_eight(dev):
+    """The runner's whole loop (zipage/engine/model_runner.py:466-469, layer_stride = 8): a
+    36-layer cache compressed as chunks of 8, 8, 8, 8 and 4 layers through the one-call entry, 32
+    ragged sequences with shared prefix pages.  Every layer is checked for the stable in-place
+    gather; three layers of two sequences are compared with the oracle end to end."""
+    from zipage_amd.compress import CompressConfig, compress_layers
+    from zipage_amd.workload import cpu_subset, ragged_batch
+    L, stride = 36, 8
+    wl = ragged_batch(32, L=L, pool_pages=400, budget=BUDGET, W=32, seed=9, lengths=(2049, 2560),
+                      shared_prefix_group=16, shared_prefix_pages=2)
+    shared = sorted({t[0] for t in wl.tables} | {t[1] for t in wl.tables})
+    kb, vb = _save_touched(wl)
+    seqs, layers = [3, 20], [0, 17, 35]
+    sub = cpu_subset(wl, seqs)
+    kw = dict(enable_pooling=True, pooling_size=7)
+    cfg = CompressConfig(budget_blocks=BUDGET, query_cache_len=32, **kw)
+    flags = []
+    for l0 in range(0, L, stride):
+        l1 = min(l0 + stride, L)
+        flags.append(compress_layers(wl.k[l0:l1], wl.v[l0:l1], wl.q[l0:l1], None, wl.query_ids,
+                                     wl.block_tables, wl.compressed, wl.targets, cfg))
+    flag = torch.cat(flags, 0)
+    assert flag.shape[0] == L and not torch.equal(flag[0], flag[L - 1])
+    _check_properties(wl, flag, None, kb, vb, shared_pages=shared)
+    # oracle, end to end, on the sampled layers (keys / queries differ per layer)
+    kk = BUDGET * BS
+    for l in layers:
+        ok, ov = sub["k"][l:l + 1].clone(), sub["v"][l:l + 1].clone()
+        oflag = O.compress_pipeline(ok, ov, sub["q"][l:l + 1], None, sub["query_ids"], sub["block_tables"],
+                                    sub["compressed"], sub["targets"], budget_blocks=BUDGET,
+                                    query_cache_len=32, **kw)
+        g = flag[l:l + 1, seqs].cpu()
+        mism = (g != oflag).float().mean().item()
+        print(f"  layer {l}: keep flags differing from the oracle's: {mism:.2e}")
+        assert mism <= 6e-3, mism
+        assert (g.view(1, len(seqs), -1, g.shape[-2] * BS).sum(-1) == kk).all()
 
 
 def test_config1_single_sequence_fp32_full_oracle(dev):
