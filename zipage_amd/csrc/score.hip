@@ -392,9 +392,8 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
               }
             }
           }
-#pragma unroll 1
-          for (; sti < NSUB; ++sti) {
-            const int st = tg * NSUB + sti;
+          // one 32 x 32 block of products: query row block x the tokens of subtile st
+          auto products = [&](int st) {
             f32x16_t acc;
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[r] = 0.f;
@@ -420,9 +419,15 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
 #pragma unroll
               for (int s = 0; s < KB; ++s) acc = M::mma(afrag[s0 + s], bfr[s], acc);
             }
+            return acc;
+          };
+          // what a sweep does with a block of products.  MASKED: the causal mask of a last page
+          // may apply (a uniform branch; the unmasked form is a single basic block)
+          auto epilogue = [&](f32x16_t acc, int st, int sti, auto masked_c) {
+            constexpr bool MASKED = decltype(masked_c)::value;
             const int slot = toff + st * 32 + col;  // token slot inside its page
             // causal mask: only the tail of the last page can be hidden from a window row
-            if (last && (toff + st * 32 + 31 > p.BS - p.W)) {
+            if (MASKED && last && (toff + st * 32 + 31 > p.BS - p.W)) {
 #pragma unroll
               for (int r = 0; r < 16; ++r) {
                 const int w = (row0 + (r >> 2) * 8 + (r & 3)) >> gsV;
@@ -549,6 +554,44 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
                 if (half == 0) part[((tile & 1) * kRowWaves + rbw) * TN + st * 32 + col] = red;
               }
             }
+                    };
+          if constexpr ((PASS == 1 || PASS == 2) && !LOGITS && T::bytes == 2) {
+            // Sum and output sweeps, whole tiles away from the causal mask: the products of subtile
+            // k+1 are issued between the epilogue instructions of subtile k, so the matrix core
+            // works while the vector unit runs the epilogue (a lone wave would do one after the other).
+            if (NSUB == 4 && !last) {
+              const int st0 = tg * 4;
+              auto interleave = [&]() {
+                __builtin_amdgcn_sched_group_barrier(0x100, KS, 0);     // the LDS reads first
+#pragma unroll
+                for (int s = 0; s < KS; ++s) {
+                  __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);    // one MFMA
+                  __builtin_amdgcn_sched_group_barrier(0x002, PASS == 1 ? 14 : 13, 0);   // a share of the epilogue
+                }
+              };
+              const std::false_type unmasked{};
+              const f32x16_t a0 = products(st0);
+              __builtin_amdgcn_sched_barrier(0);
+              const f32x16_t a1 = products(st0 + 1);
+              epilogue(a0, st0, 0, unmasked);
+              interleave();
+              __builtin_amdgcn_sched_barrier(0);
+              const f32x16_t a2 = products(st0 + 2);
+              epilogue(a1, st0 + 1, 1, unmasked);
+              interleave();
+              __builtin_amdgcn_sched_barrier(0);
+              const f32x16_t a3 = products(st0 + 3);
+              epilogue(a2, st0 + 2, 2, unmasked);
+              interleave();
+              __builtin_amdgcn_sched_barrier(0);
+              epilogue(a3, st0 + 3, 3, unmasked);
+              sti = NSUB;
+            }
+          }
+#pragma unroll 1
+          for (; sti < NSUB; ++sti) {
+            const int st = tg * NSUB + sti;
+            epilogue(products(st), st, sti, std::true_type{});
           }
         } else if (PASS == 2) {
 #pragma unroll
