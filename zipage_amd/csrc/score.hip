@@ -770,29 +770,19 @@ extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
 #define ZP_SCORE_LAUNCH()                                                                        \
   do {                                                                                           \
     const size_t smem = 2 * (size_t)Mma<T>::TN * Mma<T>::ROWB +                                  \
-                        sizeof(float) * (2 * kRowWaves * Mma<T>::TN + kWaves * 32) + sizeof(int) * 2 * NB;            \
+                        sizeof(float) * (2 * kRowWaves * Mma<T>::TN + kWaves * 32) + sizeof(int) * 2 * NB; \
+    void (*fn)(ScoreArgs) = score_kernel<T, false, 0, -1>;                                       \
+    if (logits_out) fn = score_kernel<T, true, 0, -1>;                                           \
+    else if (T::bytes == 2 && Gp == 4 && !a.reduce_max) fn = score_kernel<T, false, 4, 0>;       \
+    else if (T::bytes == 2 && Gp == 2 && !a.reduce_max) fn = score_kernel<T, false, 2, 0>;       \
+    else if (T::bytes == 2 && Gp == 8 && !a.reduce_max) fn = score_kernel<T, false, 8, 0>;       \
     if (smem > 64 * 1024 &&                                                                      \
-        (hipFuncSetAttribute((const void*)score_kernel<T, false, 0, -1>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                            (int)smem) != hipSuccess ||                                         \
-         hipFuncSetAttribute((const void*)score_kernel<T, false, 4, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                            (int)smem) != hipSuccess ||                                         \
-         hipFuncSetAttribute((const void*)score_kernel<T, false, 2, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                            (int)smem) != hipSuccess ||                                         \
-         hipFuncSetAttribute((const void*)score_kernel<T, false, 8, 0>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                            (int)smem) != hipSuccess ||                                         \
-         hipFuncSetAttribute((const void*)score_kernel<T, true, 0, -1>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                            (int)smem) != hipSuccess)) {                                          \
+        hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize,         \
+                            (int)smem) != hipSuccess) {                                          \
       zp_set_error("attention_score: cannot reserve %zu bytes of LDS", smem);                    \
       return ZP_EHIP;                                                                            \
     }                                                                                            \
-    if (logits_out) hipLaunchKernelGGL((score_kernel<T, true, 0, -1>), grid, dim3(kThreads), smem, st, a);  \
-    else if (T::bytes == 2 && Gp == 4 && !a.reduce_max)                                          \
-      hipLaunchKernelGGL((score_kernel<T, false, 4, 0>), grid, dim3(kThreads), smem, st, a);     \
-    else if (T::bytes == 2 && Gp == 2 && !a.reduce_max)                                          \
-      hipLaunchKernelGGL((score_kernel<T, false, 2, 0>), grid, dim3(kThreads), smem, st, a);     \
-    else if (T::bytes == 2 && Gp == 8 && !a.reduce_max)                                          \
-      hipLaunchKernelGGL((score_kernel<T, false, 8, 0>), grid, dim3(kThreads), smem, st, a);     \
-    else hipLaunchKernelGGL((score_kernel<T, false, 0, -1>), grid, dim3(kThreads), smem, st, a); \
+    hipLaunchKernelGGL(fn, grid, dim3(kThreads), smem, st, a);                                   \
   } while (0)
   ZP_DISPATCH_DTYPE(dtype, ZP_SCORE_LAUNCH());
 #undef ZP_SCORE_LAUNCH
