@@ -269,6 +269,23 @@ def test_attention_score(dev, dtype, cfg, reduced):
         assert torch.equal(got2, got)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("BS,D", [(128, 128), (512, 128), (256, 64), (128, 32), (384, 96)])
+def test_attention_score_head_dims_and_page_sizes(dev, dtype, BS, D):
+    """Head dims below 128 (part of every staged key row stays zero) and pages of one, two, three
+    and four 128-token tiles (the tile -> page mapping is a shift or a division)."""
+    from zipage_amd.kernel import attention_score
+    s = _setup(59, dtype, L=1, B=3, Hkv=2, Hq=8, D=D, W=32, BS=BS, nb_choices=(2, 3, 4), num_pages=20)
+    args = (s["k"], s["q"], s["seq_idx"], s["enc"])
+    want = O.attention_score(*args)
+    got = attention_score(*(a.to(dev) for a in args))
+    assert got.shape == want.shape and got.dtype == dtype
+    if dtype == torch.float32:
+        _rel_close(got, want, rel=1e-3, abs_floor=1e-9)
+    else:
+        _ulp_close(got, want, dtype, ulps=2, frac_exact=0.9)
+
+
 @pytest.mark.parametrize("boost", [1.0, 40.0, 400.0])
 def test_attention_score_fp32_logit_range(dev, boost):
     """fp32 caches take the row maximum and the row sum in one sweep, every lane against its own
