@@ -158,8 +158,7 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
   char* kbuf1 = smem + TN * ROWB;
   float* part = (float*)(smem + 2 * TN * ROWB);        // [2][kRowWaves][TN]
   float* stat = part + 2 * kRowWaves * TN;              // [kWaves][32] row statistics
-  int* vpage = (int*)(stat + kWaves * 32);             // [NB] page id of valid pages
-  int* vslot = vpage + p.NB;                           // [NB] their index in the table (bit 30: last)
+  int2* vinfo = (int2*)(stat + kWaves * 32);           // [NB] valid pages: (page id, index in the table | last << 30)
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
@@ -181,8 +180,7 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
       const unsigned long long okm = __builtin_amdgcn_ballot_w64(ok);
       if (ok) {
         const int n = __builtin_popcountll(okm & lanemask_lt());
-        vpage[n] = pid;
-        vslot[n] = lane | (page_is_last(code) ? (1 << 30) : 0);
+        vinfo[n] = make_int2(pid, lane | (page_is_last(code) ? (1 << 30) : 0));
       }
       if (lane == 0) nvalid_s = __builtin_popcountll(okm);
     }
@@ -192,8 +190,7 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
       const int code = p.table[(int64_t)b * p.NB + j];
       const int pid = page_is_pad(code) ? -1 : page_id(code);
       if (pid >= 0 && pid < p.num_pages) {
-        vpage[n] = pid;
-        vslot[n] = j | (page_is_last(code) ? (1 << 30) : 0);
+        vinfo[n] = make_int2(pid, j | (page_is_last(code) ? (1 << 30) : 0));
         ++n;
       }
     }
@@ -236,9 +233,8 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
   for (int i = 0; i < STAGE_IT; ++i)
     ld_off[i] = (uint32_t)((st_row0 + i * ROWS_PER_IT) * k_row + st_piece * 16);
 
-  auto issue_loads = [&](int tile) {
+  auto issue_loads = [&](int tile, int pid) {
     const int vp = tile_page(tile), toff = (tile - vp * tiles_per_page) * TN;
-    const int pid = __builtin_amdgcn_readfirstlane(vpage[vp]);
     const char* src = kbase + (int64_t)pid * p.k_sp * T::bytes + (int64_t)toff * k_row;
 #pragma unroll
     for (int i = 0; i < STAGE_IT; ++i) {
@@ -331,8 +327,16 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
       // The middle sweep walks the tiles backwards: it starts on the tiles the first sweep read
       // last (still in L2) and ends on those the third sweep reads first.
       auto order = [&](int i) { return PASS == 1 ? ntiles - 1 - i : i; };
+      // (page id, slot) of a tile; the entry of tile it+2 is requested a whole tile before its
+      // page id is needed, so the tile loop never waits for this LDS read
+      auto tile_info = [&](int i) { return vinfo[tile_page(order(i < ntiles ? i : ntiles - 1))]; };
+      int vs = 0;          // slot word of the current tile
+      int2 info_next = make_int2(0, 0);   // entry of tile it+1
       if (ntiles > 0) {
-        issue_loads(order(0));
+        const int2 i0 = tile_info(0);
+        vs = __builtin_amdgcn_readfirstlane(i0.y);
+        issue_loads(order(0), __builtin_amdgcn_readfirstlane(i0.x));
+        info_next = tile_info(1);
         commit_loads(kbuf0);
       }
       __syncthreads();
@@ -340,9 +344,11 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
         const int tile = order(it);
         char* cur = (it & 1) ? kbuf1 : kbuf0;
         char* nxt = (it & 1) ? kbuf0 : kbuf1;
-        if (it + 1 < ntiles) issue_loads(order(it + 1));
+        const int pid_next = __builtin_amdgcn_readfirstlane(info_next.x);
+        const int vs_next = __builtin_amdgcn_readfirstlane(info_next.y);
+        info_next = tile_info(it + 2);
+        if (it + 1 < ntiles) issue_loads(order(it + 1), pid_next);
         const int vp = tile_page(tile), toff = (tile - vp * tiles_per_page) * TN;
-        const int vs = __builtin_amdgcn_readfirstlane(vslot[vp]);
         const int j = vs & 0xffff;
         const bool last = (vs >> 30) & 1;
         if (active) {
@@ -603,6 +609,7 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
         // the window partials of this tile are complete: combine the waves' shares while the
         // next tile is being computed (the buffer is rewritten two tiles later)
         if constexpr (PASS == 2) finish_tile(tile, j, toff);
+        vs = vs_next;
       }
       // the xor butterfly leaves the row result in all 32 lanes that share the row; the
       // token-group waves that share a row block then combine their halves through LDS
@@ -770,7 +777,7 @@ extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
 #define ZP_SCORE_LAUNCH()                                                                        \
   do {                                                                                           \
     const size_t smem = 2 * (size_t)Mma<T>::TN * Mma<T>::ROWB +                                  \
-                        sizeof(float) * (2 * kRowWaves * Mma<T>::TN + kWaves * 32) + sizeof(int) * 2 * NB; \
+                        sizeof(float) * (2 * kRowWaves * Mma<T>::TN + kWaves * 32) + sizeof(int2) * NB; \
     void (*fn)(ScoreArgs) = score_kernel<T, false, 0, -1>;                                       \
     if (logits_out) fn = score_kernel<T, true, 0, -1>;                                           \
     else if (T::bytes == 2 && Gp == 4 && !a.reduce_max) fn = score_kernel<T, false, 4, 0>;       \
