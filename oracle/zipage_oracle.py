@@ -13,10 +13,15 @@ rounds at exactly those points; ``rounding="fp32"`` keeps every intermediate in 
 rounds only the returned tensor.  With fp32 caches both modes are identical.
 
 Pinning status (which independent check fixes each function) lives in the tests:
-``tests/test_oracle_*.py``.  Parts that only an execution of the reference could pin
-(the precise low-precision rounding points for bf16/fp16 inputs and ``torch.topk``'s tie
-order on a GPU) are "parity unpinned": for those this file *defines* the contract
-(rounding as written below, ties broken towards the lowest index).
+``tests/test_oracle_pins.py`` (fp32: brute force, library routines, closed forms) and
+``tests/test_oracle_pins_16bit.py`` (bf16/fp16: the torch-op epilogues of the reference run as
+library ops on cache-dtype CPU tensors, bit for bit, with a mutation check per rounding).
+Parity unpinned -- only an execution of the reference on its own GPU stack could pin these, so
+this file *defines* them: ``torch.topk``'s tie order (here: lowest index first); the
+arithmetic of Triton's ``tl.dot`` on fp32 operands (TF32 on NVIDIA; here IEEE fp32); whether
+Triton rounds ``cache * decay_factor`` to the cache dtype before the max / add of
+``global_score`` (here: the product stays fp32); and that torch's GPU kernel for
+``tensor.div_(python_scalar)`` may multiply by the reciprocal (here: a true division).
 
 Page-table encoding (``zipage/engine/model_runner.py:437-463``): an int32 row per
 sequence; ``id >= 0`` is a full page, ``-1`` is padding, ``x < -1`` marks the sequence's
