@@ -259,14 +259,16 @@ def test_attention_score(dev, dtype, cfg, reduced):
         # one logit that rounds the other way moves its probability by exp(ulp(logit)), a
         # few output ulps; the window mean dilutes that, the window max does not
         _ulp_close(got, want, dtype, ulps=2 if reduced == "mean" else 16, frac_exact=0.9)
-    # without logits the scores are the same bits (fp32 caches: the same to 1e-5, because only the
-    # logit-free path takes the row maximum and the row sum in one sweep)
+    # without logits another kernel runs: fp32 caches take the row maximum and the row sum in one
+    # sweep (the same to 1e-5); 16-bit caches keep the rounded logits in registers and sweep K
+    # once -- the same rounding points, another fp32 summation order of the row sums
     got2 = attention_score(*(a.to(dev) for a in args), reduced=reduced)
     if dtype == torch.float32:
         _rel_close(got2, got, rel=1e-5, abs_floor=1e-12)
         _rel_close(got2, want, rel=1e-3, abs_floor=1e-9)
     else:
-        assert torch.equal(got2, got)
+        _ulp_close(got2, want, dtype, ulps=2 if reduced == "mean" else 16, frac_exact=0.9)
+        _ulp_close(got2, got.cpu(), dtype, ulps=2 if reduced == "mean" else 16, frac_exact=0.97)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

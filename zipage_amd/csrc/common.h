@@ -30,6 +30,11 @@ void zp_set_error(const char* fmt, ...);
     }                                                                  \
   } while (0)
 
+// Scratch zp_attention_score cannot do without (it takes the three-sweep kernel when the caller
+// brings less than zp_attention_score_workspace() asks for).  Library-internal.
+int64_t zp_attention_score_workspace_floor(int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
+                                           int32_t Hq, int32_t W);
+
 // ---------------------------------------------------------------- element types
 // Storage element tags.  bf16/fp16 are kept as raw 16-bit patterns in memory.
 struct BF16 { typedef uint16_t raw; static constexpr int bytes = 2; };

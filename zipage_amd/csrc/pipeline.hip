@@ -26,8 +26,10 @@ struct Plan {
 // Rows the one-launch selection holds in LDS (zp_select_topk's own limit).
 inline bool select_fits(int64_t Tn) { return Tn * 8 <= 150 * 1024; }
 
+// lean: give the scorer only the scratch it cannot do without (it then sweeps K three times
+// instead of keeping the logits in registers) -- for callers with a fixed scratch budget.
 Plan make_plan(int L, int B, int NB, int BS, int Hkv, int Hq, int W, int dtype,
-               const zp_compress_config* c, bool own_flag) {
+               const zp_compress_config* c, bool own_flag, bool lean = false) {
   Plan p;
   const int64_t n = (int64_t)L * B * Hkv * NB * BS;
   const int64_t es = zp_dtype_bytes(dtype);
@@ -42,7 +44,9 @@ Plan make_plan(int L, int B, int NB, int BS, int Hkv, int Hq, int W, int dtype,
                   ? take(n * es) : -1;
   p.red = c->use_redundancy ? take(n * es) : -1;
   p.flag = own_flag ? take(n) : -1;
-  p.score_ws_bytes = zp_attention_score_workspace(L, B, NB, BS, Hkv, Hq, W);
+  p.score_ws_bytes = (lean || dtype == ZP_F32)
+                         ? zp_attention_score_workspace_floor(L, B, NB, BS, Hkv, Hq, W)
+                         : zp_attention_score_workspace(L, B, NB, BS, Hkv, Hq, W);
   p.score_ws = p.score_ws_bytes ? take(p.score_ws_bytes) : -1;
   p.raw_ws_bytes = (c->use_redundancy && !c->lightning) ? zp_redundancy_raw_workspace(L, B, NB, BS, Hkv) : 0;
   p.raw_ws = p.raw_ws_bytes ? take(p.raw_ws_bytes) : -1;
@@ -281,7 +285,9 @@ extern "C" int zp_compress_layers_static(void* k_cache, void* v_cache, const voi
   ZP_REQUIRE(k_cache && v_cache && query_cache && seq_idx && block_table && compressed &&
                  target_block_table && strides, "compress_layers_static: null pointer");
   if (L == 0 || B == 0) return ZP_OK;
-  const Plan p = make_plan(L, B, NB, BS, Hkv, Hq, W, dtype, cfg, flag_out == nullptr);
+  Plan p = make_plan(L, B, NB, BS, Hkv, Hq, W, dtype, cfg, flag_out == nullptr);
+  if (p.total > (int64_t)ZP_STATIC_SCRATCH_BYTES)
+    p = make_plan(L, B, NB, BS, Hkv, Hq, W, dtype, cfg, flag_out == nullptr, true);
   ZP_REQUIRE(p.total <= (int64_t)ZP_STATIC_SCRATCH_BYTES,
              "compress_layers_static: this chunk needs %lld bytes of scratch, the library's array "
              "holds %lld; split the batch or the layers, or use zp_compress_layers with a "

@@ -80,6 +80,8 @@ struct ScoreArgs {
   int RB;  // row blocks of 32
   int gs;  // log2(Gp)
   int RW;  // waves along the row axis: 1, 2 or 4
+  float* part;    // register-resident kernel: fp32 window partials (L*B*Hkv, RB, NB*BS)
+  int n_items;    // L*B*Hkv
 };
 
 template <typename T>
@@ -699,6 +701,392 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
   }
 }
 
+
+// ================================================================ register-resident scorer
+// For 16-bit caches and sequences of at most kResTiles x 128 tokens the three sweeps collapse into
+// ONE sweep over K: the rounded logits of a block of 32 query rows stay in registers, two per
+// 32-bit word, and the row maximum, the row sum and the output are computed from the registers.
+//
+// A workgroup is one (layer, sequence, kv head, block of 32 query rows) unit; its four waves split
+// the tokens: wave t owns tokens [128 i + 32 t, 128 i + 32 t + 32) of every 128-token tile i, i.e.
+// 8 words per tile and lane.  Every wave streams its own 32-row K blocks from global memory
+// straight into LDS (no staging registers, no workgroup barrier in the sweep) two blocks ahead.
+// The row maxima and sums of the four waves meet in LDS (two barriers per unit).  The window
+// reduction of a unit covers only its own windows, so a unit writes fp32 partial sums and
+// score_combine_kernel adds the units of a (layer, sequence, head) in a fixed order, divides by
+// the window length and rounds -- the same arithmetic, in the same order, as the three-sweep
+// kernel's combine across its row-block waves.
+//
+// LDS layout of a 32-row block (rows of 256 bytes = 16 pieces of 16 bytes): a load instruction
+// fills 1 KB of consecutive LDS with four rows, so padding can only go between groups of four rows.
+// Inside a group piece g of row r sits at (g / 4) * 256 + r * 64 + (g % 4) * 16 and groups are
+// 1040 bytes apart: the sixteen lanes that read the same piece of sixteen consecutive rows then
+// fall into sixteen different 16-byte bank groups, a quad of lanes still fetches 64 consecutive
+// bytes of one row, and the fragment of contraction step s is an immediate offset from one base.
+constexpr int kResTiles = 20;
+constexpr int kGrp = 1040;
+constexpr int kSubBytes = 8 * kGrp;
+
+template <typename T> struct Pack2;
+template <> struct Pack2<BF16> {
+  __device__ static __forceinline__ uint32_t pack(float lo, float hi) {
+    typedef __attribute__((ext_vector_type(2))) float f2;
+    typedef __attribute__((ext_vector_type(2))) __bf16 b2;
+    const f2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, b2));
+  }
+  __device__ static __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
+  __device__ static __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+};
+template <> struct Pack2<F16> {
+  typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+  __device__ static __forceinline__ uint32_t pack(float lo, float hi) {
+    const h2 v = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+  }
+  __device__ static __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(h2, w)[0]; }
+  __device__ static __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(h2, w)[1]; }
+};
+
+// Group maximum and window reduction of the sixteen exponents a lane holds for one token
+// (pv[r] = x log2(e) - log2(row sum), rows (r/4)*8 + half*4 + r%4 of the block): the probability
+// is 2^pv rounded to the cache dtype; exponential and rounding are monotone, so the maximum over
+// the group is taken first.  Returns the lane's share of the window sum (or maximum) over the
+// windows of the block, both wave halves already combined when they hold different windows.
+template <typename T>
+__device__ __forceinline__ float group_window_reduce(float (&pv)[16], int Gp, bool rmaxV) {
+  float red;
+  if (Gp < 2) {
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      pv[r] = exp2_hw(pv[r]);
+      pv[r + 1] = exp2_hw(pv[r + 1]);
+      Rnd<T>::pair(pv[r], pv[r + 1]);
+    }
+  }
+  if (Gp >= 4) {
+    float q4[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      q4[q] = vmax(vmax(pv[4 * q], pv[4 * q + 1]), vmax(pv[4 * q + 2], pv[4 * q + 3]));
+    if (Gp >= 8) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) q4[q] = vmax(q4[q], lane_xor32(q4[q]));
+    }
+    if (Gp < 16) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) q4[q] = exp2_hw(q4[q]);
+      Rnd<T>::pair(q4[0], q4[1]);
+      Rnd<T>::pair(q4[2], q4[3]);
+    }
+    if (Gp >= 16) {
+      q4[0] = vmax(q4[0], q4[1]);
+      q4[2] = vmax(q4[2], q4[3]);
+      if (Gp >= 32) {
+        red = exp2_hw(vmax(q4[0], q4[2]));
+        float dummy = red;
+        Rnd<T>::pair(red, dummy);
+      } else {
+        q4[0] = exp2_hw(q4[0]);
+        q4[2] = exp2_hw(q4[2]);
+        Rnd<T>::pair(q4[0], q4[2]);
+        red = rmaxV ? vmax(q4[0], q4[2]) : q4[0] + q4[2];
+      }
+    } else {
+      red = rmaxV ? vmax(vmax(q4[0], q4[1]), vmax(q4[2], q4[3])) : (q4[0] + q4[1]) + (q4[2] + q4[3]);
+    }
+  } else {
+    float t8[8];
+    if (Gp == 2) {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) t8[q] = exp2_hw(vmax(pv[2 * q], pv[2 * q + 1]));
+#pragma unroll
+      for (int q = 0; q < 8; q += 2) Rnd<T>::pair(t8[q], t8[q + 1]);
+    } else {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) t8[q] = rmaxV ? vmax(pv[2 * q], pv[2 * q + 1]) : pv[2 * q] + pv[2 * q + 1];
+    }
+    if (rmaxV) {
+      red = vmax(vmax(vmax(t8[0], t8[1]), vmax(t8[2], t8[3])), vmax(vmax(t8[4], t8[5]), vmax(t8[6], t8[7])));
+    } else {
+      red = ((t8[0] + t8[1]) + (t8[2] + t8[3])) + ((t8[4] + t8[5]) + (t8[6] + t8[7]));
+    }
+  }
+  if (Gp < 8) {  // the two lane halves hold different windows
+    const float o = lane_xor32(red);
+    red = rmaxV ? vmax(red, o) : red + o;
+  }
+  return red;
+}
+
+// TPP: 128-token tiles per page when known at compile time (0: from the arguments); with it
+// the page of every unrolled tile is a constant and its id comes from a lane of a register.
+template <typename T, int GPC, int RMAXC, int TPP>
+__global__ __launch_bounds__(kThreads, 2) void score_resident_kernel(ScoreArgs p) {
+  typedef Mma<T> M;
+  typedef typename M::Frag Frag;
+  typedef Pack2<T> P2;
+  constexpr int KS = M::KS;   // 8 contraction steps of 16
+  const int GpV = GPC > 0 ? GPC : p.Gp;
+  const int gsV = GPC == 8 ? 3 : GPC == 4 ? 2 : GPC == 2 ? 1 : p.gs;
+  const bool rmaxV = RMAXC >= 0 ? (RMAXC != 0) : (p.reduce_max != 0);
+
+  extern __shared__ __align__(16) char smem[];
+  float* stat = (float*)(smem + kWaves * 2 * kSubBytes);   // [kWaves][32]
+  int2* vinfo = (int2*)(stat + kWaves * 32);               // [NB]
+  __shared__ int nvalid_s;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5, col = lane & 31;
+  // unit -> (item, row block): workgroup ids are dealt round-robin to the 8 XCDs; the row blocks
+  // of an item get consecutive ids ON ONE XCD, so they run at the same time behind one L2 and
+  // the item's keys leave HBM once
+  const int xcd = blockIdx.x & 7, loc = blockIdx.x >> 3;
+  const int rb = loc % p.RB;
+  const int item = (loc / p.RB) * 8 + xcd;
+  if (item >= p.n_items) return;
+  const int h = item % p.Hkv;
+  const int b = (item / p.Hkv) % p.B;
+  const int l = item / (p.Hkv * p.B);
+  const int Tn = p.NB * p.BS;
+
+  if (wave == 0) {
+    const int code = lane < p.NB ? p.table[(int64_t)b * p.NB + lane] : -1;
+    const int pid = page_is_pad(code) ? -1 : page_id(code);
+    const bool ok = pid >= 0 && pid < p.num_pages;
+    const unsigned long long okm = __builtin_amdgcn_ballot_w64(ok);
+    if (ok) {
+      const int n = __builtin_popcountll(okm & lanemask_lt());
+      vinfo[n] = make_int2(pid, lane | (page_is_last(code) ? (1 << 30) : 0));
+    }
+    if (lane == 0) nvalid_s = __builtin_popcountll(okm);
+  }
+  const int dpieces = p.D * T::bytes / 16;
+  char* kb = smem + wave * 2 * kSubBytes;    // this wave's two K blocks
+  if (dpieces < 16)   // the tail of every staged row must read as zero
+    for (int i = lane; i < 2 * kSubBytes / 4; i += 64) ((uint32_t*)kb)[i] = 0u;
+  __syncthreads();
+  const int nvalid = nvalid_s;
+  // lane j keeps entry j of the valid-page list: (page id, table index | last << 30)
+  const int2 myinfo = lane < nvalid ? vinfo[lane] : make_int2(0, 0);
+  int seq = p.seq_idx[b];
+  const bool seq_ok = seq >= 0 && seq < p.max_seqs;
+  if (!seq_ok) seq = 0;
+
+  const int tiles_per_page = TPP > 0 ? TPP : p.BS / 128;
+  const int ntiles = nvalid * tiles_per_page;
+  auto tile_page = [&](int tile) { return TPP > 0 ? tile / TPP : tile / tiles_per_page; };
+  auto page_word = [&](int v, int vp) {   // entry vp of the list, wave-uniform
+    if constexpr (TPP > 0) return __builtin_amdgcn_readlane(v, vp);
+    else return __builtin_amdgcn_readfirstlane(__builtin_amdgcn_ds_bpermute(vp << 2, v));
+  };
+  const int64_t k_row = (int64_t)p.Hkv * p.D * T::bytes;
+  const char* kbase = p.k + (l * p.k_sl) * T::bytes + (int64_t)h * p.D * T::bytes;
+  const int wtok = wave * 32;   // this wave's tokens inside a tile
+
+  // ---- staging: a load instruction moves four rows; lane -> (row of the group, piece).  The
+  // rows go through a buffer descriptor based at the block's first row, so an instruction needs
+  // one fixed per-lane offset, a scalar offset and no address arithmetic.
+  const int st_g = (lane >> 4) * 4 + (lane & 3), st_r = (lane >> 2) & 3;
+  const int st_off = (int)(st_r * k_row + st_g * 16);
+  const bool st_ok = st_g < dpieces;
+  const int grp_step = (int)(4 * k_row);
+  typedef void __attribute__((address_space(3))) * lptr_t;
+  auto issue = [&](int tile, char* buf) {
+    const int vp = tile_page(tile);
+    const int pid = page_word(myinfo.x, vp);
+    const int toff = (tile - vp * tiles_per_page) * 128 + wtok;
+    const char* src = kbase + (int64_t)pid * p.k_sp * T::bytes + (int64_t)toff * k_row;
+    const __amdgpu_buffer_rsrc_t rs =
+        __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, (int)(32 * k_row), 0x00020000);
+    if (st_ok) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lptr_t)(buf + i * kGrp), 16, st_off,
+                                                 i * grp_step, 0, 0);
+    }
+  };
+  // fragment of step s of this lane's row: base + (s / 2) * 256 + (s % 2) * 32
+  const int rd_off = (col >> 2) * kGrp + (col & 3) * 64 + half * 16;
+
+  if (ntiles > 0) issue(0, kb);
+  if (ntiles > 1) issue(1, kb + kSubBytes);
+
+  // ---- A fragments: the 32 query rows of this block, in registers for the whole sweep
+  Frag afrag[KS];
+  {
+    const int mrow = rb * 32 + col;
+    const int a_w = mrow >> gsV, a_g = mrow & (GpV - 1);
+    const bool a_ok = seq_ok && a_w < p.W && a_g < p.G;
+    const char* qrow = p.q + ((int64_t)l * p.q_sl + (int64_t)seq * p.q_ss +
+                              ((int64_t)a_w * p.Hq + (int64_t)h * p.G + a_g) * p.D) * T::bytes;
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int k0 = s * M::KPI + half * M::EPL;
+      if (a_ok && k0 < p.D) afrag[s] = *(const Frag*)(qrow + (int64_t)k0 * T::bytes);
+      else zero_frag<T>(afrag[s]);
+    }
+  }
+  // the sweep counts its own loads with s_waitcnt: the query loads must be out of the way.  They
+  // were issued after the first two K blocks, so waiting for them waits for those blocks too.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(afrag[s]));
+
+  const int row0 = rb * 32 + half * 4;   // rows of this lane: row0 + (r/4)*8 + r%4
+  uint32_t lg[kResTiles * 8];
+  float run[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) run[r] = -INFINITY;
+
+  // ---- the sweep: products, causal mask, running maximum, rounded logits into registers
+#pragma unroll
+  for (int it = 0; it < kResTiles; ++it) {
+    if (it < ntiles) {
+      // block `it` has landed once at most the 8 loads of block it+1 are outstanding
+      if (it >= 2) {
+        if (it + 1 < ntiles) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      const char* cur = kb + (it & 1) * kSubBytes + rd_off;
+      f32x16_t acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+      for (int s0 = 0; s0 < KS; s0 += 4) {
+        Frag bfr[4];
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+          bfr[s] = *(const Frag*)(cur + ((s0 + s) >> 1) * 256 + ((s0 + s) & 1) * 32);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) acc = M::mma(afrag[s0 + s], bfr[s], acc);
+      }
+      // every fragment of this buffer is in registers: block it+2 may overwrite it
+      asm volatile("" ::: "memory");
+      if (it + 2 < ntiles) issue(it + 2, kb + (it & 1) * kSubBytes);
+      const int vp = tile_page(it);
+      const int vs = page_word(myinfo.y, vp);
+      const int toff = (it - vp * tiles_per_page) * 128 + wtok;
+      if (((vs >> 30) & 1) && (toff + 31 > p.BS - p.W)) {   // causal mask: tail of the last page
+        const int slot = toff + col;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int w = (row0 + (r >> 2) * 8 + (r & 3)) >> gsV;
+          if (slot > p.BS - p.W + w) acc[r] = -INFINITY;
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 16; ++r) run[r] = vmax(run[r], acc[r]);
+#pragma unroll
+      for (int r = 0; r < 16; r += 2)
+        lg[it * 8 + (r >> 1)] = P2::pack(acc[r] * p.scale, acc[r + 1] * p.scale);
+    }
+  }
+
+  // ---- row maximum over the lanes of a row and the four waves
+  auto row_slot = [&](int r) { return (r >> 2) * 8 + half * 4 + (r & 3); };
+  float mx[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const float v = half_max(run[r]);
+    run[r] = v;
+    if (col == 0) stat[wave * 32 + row_slot(r)] = v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float v = run[r];
+#pragma unroll
+    for (int w2 = 1; w2 < kWaves; ++w2) v = fmaxf(v, stat[((wave + w2) % kWaves) * 32 + row_slot(r)]);
+    mx[r] = Elem<T>::rnd(v * p.scale);
+  }
+  __syncthreads();
+
+  // ---- x = rounded(logit - max) back into the registers, row sums of exp(x)
+#pragma unroll
+  for (int r = 0; r < 16; ++r) run[r] = 0.f;
+#pragma unroll
+  for (int it = 0; it < kResTiles; ++it) {
+    if (it < ntiles) {
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const uint32_t w = lg[it * 8 + q];
+        const uint32_t x = P2::pack(P2::lo(w) - mx[2 * q], P2::hi(w) - mx[2 * q + 1]);
+        lg[it * 8 + q] = x;
+        run[2 * q] += exp_neg(P2::lo(x));
+        run[2 * q + 1] += exp_neg(P2::hi(x));
+      }
+    }
+  }
+  float cl[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const float v = half_sum(run[r]);
+    run[r] = v;
+    if (col == 0) stat[wave * 32 + row_slot(r)] = v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    // the four waves' sums are added in wave order, whichever wave does it
+    float v = stat[row_slot(r)];
+#pragma unroll
+    for (int w2 = 1; w2 < kWaves; ++w2) v += stat[w2 * 32 + row_slot(r)];
+    const int m = row0 + (r >> 2) * 8 + (r & 3);
+    const bool ok = (m >> gsV) < p.W && (m & (GpV - 1)) < p.G;
+    cl[r] = ok ? -__builtin_amdgcn_logf(v) : -INFINITY;   // rows outside the window or group never win a maximum
+  }
+
+  // ---- output: p = 2^(x log2(e) - log2(sum)), group maximum, this block's share of the window sum
+  float* part = p.part + ((int64_t)item * p.RB + rb) * Tn + wtok + col;
+#pragma unroll
+  for (int it = 0; it < kResTiles; ++it) {
+    if (it < ntiles) {
+      float pv[16];
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const uint32_t x = lg[it * 8 + q];
+        pv[2 * q] = __builtin_fmaf(P2::lo(x), 1.44269504088896340736f, cl[2 * q]);
+        pv[2 * q + 1] = __builtin_fmaf(P2::hi(x), 1.44269504088896340736f, cl[2 * q + 1]);
+      }
+      const float red = group_window_reduce<T>(pv, GpV, rmaxV);
+      const int vp = tile_page(it);
+      const int j = page_word(myinfo.y, vp) & 0xffff;
+      const int toff = (it - vp * tiles_per_page) * 128;
+      if (half == 0) __builtin_nontemporal_store(red, part + j * p.BS + toff);
+    }
+  }
+}
+
+// Adds the row blocks' window partials of every (layer, sequence, head) in block order, divides by
+// the window length, rounds to the cache dtype; pad pages score exactly 0.
+template <typename T>
+__global__ __launch_bounds__(256) void score_combine_kernel(const float* __restrict__ part,
+                                                            void* __restrict__ out,
+                                                            const int32_t* __restrict__ table,
+                                                            int B, int NB, int BS, int Hkv, int RB,
+                                                            int W, int num_pages, int rmax) {
+  const int item = blockIdx.x;
+  const int b = (item / Hkv) % B;
+  const int Tn = NB * BS;
+  const int t = blockIdx.y * 256 + threadIdx.x;
+  if (t >= Tn) return;
+  const int code = table[(int64_t)b * NB + t / BS];
+  const int pid = page_is_pad(code) ? -1 : page_id(code);
+  float v = 0.f;
+  if (pid >= 0 && pid < num_pages) {
+    const float* src = part + (int64_t)item * RB * Tn + t;
+    v = __builtin_nontemporal_load(src);
+    for (int r = 1; r < RB; ++r) {
+      const float o = __builtin_nontemporal_load(src + (int64_t)r * Tn);
+      v = rmax ? fmaxf(v, o) : v + o;
+    }
+    if (!rmax) v = Elem<T>::rnd(v / (float)W);
+  }
+  Elem<T>::st(out, (int64_t)item * Tn + t, v);
+}
+
 }  // namespace
 
 static int pow2_ceil(int v) {
@@ -707,13 +1095,38 @@ static int pow2_ceil(int v) {
   return p;
 }
 
-extern "C" int64_t zp_attention_score_workspace(int32_t L, int32_t B, int32_t NB, int32_t BS,
-                                                int32_t Hkv, int32_t Hq, int32_t W) {
-  if (Hkv <= 0 || Hq <= 0) return 0;
+// Can the register-resident kernel take this shape (16-bit caches only; the caller checks the
+// dtype, the logits request and the sign of the scale)?
+static bool resident_shape_ok(int NB, int BS, int Hkv, int Hq, int D) {
+  if (Hkv <= 0 || Hq <= 0 || Hq % Hkv != 0) return false;
+  const int Gp = pow2_ceil(Hq / Hkv);
+  return BS % 128 == 0 && (int64_t)NB * (BS / 128) <= kResTiles && NB <= 64 && Gp <= 32 &&
+         D <= kDmax && (D * 2) % 16 == 0;
+}
+
+// Scratch the three-sweep kernel cannot do without (window x group beyond 128 rows).
+static int64_t sweep_workspace(int L, int B, int NB, int BS, int Hkv, int Hq, int W) {
   const int Gp = pow2_ceil(Hq / Hkv);
   const int RB = (W * Gp + 31) / 32;
   if (RB <= kRowWaves) return 0;
   return (int64_t)L * B * Hkv * NB * BS * 4;
+}
+
+extern "C" int64_t zp_attention_score_workspace(int32_t L, int32_t B, int32_t NB, int32_t BS,
+                                                int32_t Hkv, int32_t Hq, int32_t W) {
+  if (Hkv <= 0 || Hq <= 0 || L < 0 || B < 0 || NB <= 0 || BS <= 0 || W <= 0) return 0;
+  const int64_t floor_bytes = sweep_workspace(L, B, NB, BS, Hkv, Hq, W);
+  if (!resident_shape_ok(NB, BS, Hkv, Hq, kDmax)) return floor_bytes;
+  const int Gp = pow2_ceil(Hq / Hkv);
+  const int64_t RB = (W * Gp + 31) / 32;
+  const int64_t res = (int64_t)L * B * Hkv * RB * NB * BS * 4;   // fp32 window partials per row block
+  return res > floor_bytes ? res : floor_bytes;
+}
+
+int64_t zp_attention_score_workspace_floor(int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
+                                           int32_t Hq, int32_t W) {
+  if (Hkv <= 0 || Hq <= 0) return 0;
+  return sweep_workspace(L, B, NB, BS, Hkv, Hq, W);
 }
 
 extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
@@ -756,8 +1169,15 @@ extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
   ZP_REQUIRE(NB <= 0xffff, "attention_score: too many pages per sequence");
   if (L == 0 || B == 0) return ZP_OK;
   const int RB = (W * Gp + 31) / 32;
-  const int64_t need = zp_attention_score_workspace(L, B, NB, BS, Hkv, Hq, W);
-  ZP_REQUIRE(need == 0 || (workspace && workspace_bytes >= need),
+  const int64_t need = sweep_workspace(L, B, NB, BS, Hkv, Hq, W);
+  // One sweep over K with the logits in registers when the shape allows it and the caller
+  // brought the scratch for the window partials; three sweeps otherwise.
+  const int64_t res_need = (int64_t)L * B * Hkv * RB * NB * BS * 4;
+  const bool resident = es == 2 && !logits_out && softmax_scale > 0.f &&
+                        resident_shape_ok(NB, BS, Hkv, Hq, D) && workspace &&
+                        workspace_bytes >= res_need && ((uintptr_t)workspace % 4) == 0 &&
+                        (int64_t)L * B * Hkv < ((int64_t)1 << 28);
+  ZP_REQUIRE(resident || need == 0 || (workspace && workspace_bytes >= need),
              "attention_score: workspace of %lld bytes required", (long long)need);
 
   ScoreArgs a;
@@ -773,6 +1193,31 @@ extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
   if (a.RW < kWaves / (TN / 32)) a.RW = kWaves / (TN / 32);  // every wave needs >= 1 subtile
 
   hipStream_t st = (hipStream_t)stream;
+  a.n_items = L * B * Hkv;
+  a.part = (float*)workspace;
+  if (resident) {
+    const size_t smem = (size_t)kWaves * 2 * kSubBytes + sizeof(float) * kWaves * 32 + sizeof(int2) * NB;
+    const unsigned units = (unsigned)(((int64_t)a.n_items + 7) / 8 * 8 * RB);
+    const dim3 cgrid((unsigned)a.n_items, (unsigned)((NB * BS + 255) / 256));
+#define ZP_RESIDENT_LAUNCH(TT)                                                                   \
+  do {                                                                                           \
+    void (*fn)(ScoreArgs) = score_resident_kernel<TT, 0, -1, 0>;                                 \
+    if (Gp == 4 && !a.reduce_max && BS == 256) fn = score_resident_kernel<TT, 4, 0, 2>;          \
+    if (hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize,         \
+                            (int)smem) != hipSuccess) {                                          \
+      zp_set_error("attention_score: cannot reserve %zu bytes of LDS", smem);                    \
+      return ZP_EHIP;                                                                            \
+    }                                                                                            \
+    hipLaunchKernelGGL(fn, dim3(units), dim3(kThreads), smem, st, a);                            \
+    hipLaunchKernelGGL(score_combine_kernel<TT>, cgrid, dim3(256), 0, st, a.part, scores_out,    \
+                       block_table, B, NB, BS, Hkv, RB, W, num_pages, a.reduce_max);             \
+  } while (0)
+    if (dtype == ZP_BF16) ZP_RESIDENT_LAUNCH(BF16);
+    else ZP_RESIDENT_LAUNCH(F16);
+#undef ZP_RESIDENT_LAUNCH
+    ZP_LAUNCH_CHECK();
+    return ZP_OK;
+  }
   dim3 grid((unsigned)((int64_t)L * B * Hkv));
 #define ZP_SCORE_LAUNCH()                                                                        \
   do {                                                                                           \
