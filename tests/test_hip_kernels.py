@@ -307,6 +307,63 @@ def test_attention_score_fp32_logit_range(dev, boost):
     assert torch.isfinite(got.float()).all()
 
 
+def _score_three_sweeps(k, q, seq_idx, enc, reduced="mean"):
+    """zp_attention_score without the scratch for the window partials: the library then takes
+    the kernel that sweeps K three times."""
+    from zipage_amd import _lib
+    L, P, BS, Hkv, D = k.shape
+    _, S, W, Hq, _ = q.shape
+    B, NB = enc.shape
+    lib = _lib.load()
+    out = torch.empty((L, B, Hkv, NB, BS), device=k.device, dtype=k.dtype)
+    assert lib.zp_attention_score_workspace(L, B, NB, BS, Hkv, Hq, W) > 0
+    _lib.call("zp_attention_score", _lib.dev_ptr(k), _lib.dev_ptr(q), _lib.dev_ptr(seq_idx),
+              _lib.dev_ptr(enc), _lib.dev_ptr(out), 0, L, B, NB, BS, Hkv, Hq, D, W, P, S,
+              k.stride(0), k.stride(1), q.stride(0), q.stride(1), float(D ** -0.5),
+              {"mean": 0, "max": 1}[reduced], _lib.dtype_tag(k), 0, 0, _lib.stream_ptr(k))
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [
+    dict(Hkv=2, Hq=8, W=32, nb_choices=(9, 10)),            # four row blocks, 18-20 tiles
+    dict(Hkv=2, Hq=8, W=16, nb_choices=(2, 5, 9)),          # two row blocks
+    dict(Hkv=1, Hq=7, W=24, nb_choices=(3, 4)),             # group 7 padded to 8: six row blocks
+    dict(Hkv=3, Hq=3, W=8, nb_choices=(1, 2)),              # no group, a quarter of a row block
+    dict(Hkv=2, Hq=4, W=32, D=64, BS=128, nb_choices=(7, 20)),   # one tile per page, 64-wide heads
+    dict(Hkv=2, Hq=8, W=32, BS=384, nb_choices=(2, 6)),     # three tiles per page
+])
+@pytest.mark.parametrize("reduced", ["mean", "max"])
+def test_attention_score_one_sweep_matches_three_sweeps(dev, dtype, shape, reduced):
+    """16-bit caches, sequences of at most 2560 tokens: the kernel that keeps the rounded logits
+    in registers (one sweep over K) against the three-sweep kernel and against the oracle.  Same
+    rounding points; the row sums are added in another order, which moves a few values across a
+    rounding boundary."""
+    from zipage_amd.kernel import attention_score
+    shape = dict(shape)
+    nb = shape.pop("nb_choices")
+    s = _setup(71, dtype, L=2, B=4, nb_choices=nb, num_pages=48, **shape)
+    args = tuple(a.to(dev) for a in (s["k"], s["q"], s["seq_idx"], s["enc"]))
+    one = attention_score(*args, reduced=reduced)
+    three = _score_three_sweeps(*args, reduced=reduced)
+    ulps = 2 if reduced == "mean" else 16
+    _ulp_close(one, three.cpu(), dtype, ulps=ulps, frac_exact=0.98)
+    want = O.attention_score(s["k"], s["q"], s["seq_idx"], s["enc"], reduced=reduced)
+    _ulp_close(one, want, dtype, ulps=ulps, frac_exact=0.9)
+    pad = (s["enc"] == -1).view(1, -1, 1, s["enc"].shape[1], 1).expand_as(want)
+    assert (one.cpu()[pad] == 0).all()     # pad pages score exactly 0
+
+
+def test_attention_score_long_rows_take_three_sweeps(dev):
+    """More than 2560 tokens do not fit the registers: same entry point, three sweeps."""
+    from zipage_amd.kernel import attention_score
+    dtype = torch.bfloat16
+    s = _setup(73, dtype, L=1, B=2, Hkv=2, Hq=8, W=32, nb_choices=(11, 12), num_pages=32)
+    args = (s["k"], s["q"], s["seq_idx"], s["enc"])
+    got = attention_score(*(a.to(dev) for a in args))
+    _ulp_close(got, O.attention_score(*args), dtype, ulps=2, frac_exact=0.9)
+
+
 def test_attention_score_reference_script_shape(dev):
     """Shape of the reference's own script: 2 seqs, tables [[0,1,2,-5],[5,6,-9,-1]], W=24,
     Hq=16, Hkv=2, D=128, fp16 (tests/test_attention_score.py:314-358)."""

@@ -833,12 +833,22 @@ __global__ __launch_bounds__(kThreads, 2) void score_resident_kernel(ScoreArgs p
 
   extern __shared__ __align__(16) char smem[];
   float* stat = (float*)(smem + kWaves * 2 * kSubBytes);   // [kWaves][32]
-  int2* vinfo = (int2*)(stat + kWaves * 32);               // [NB]
-  __shared__ int nvalid_s;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, col = lane & 31;
+#ifdef ZP_RES_STAMP
+  // Measurement build: wave 0 of every unit records the core-clock counter at the phase
+  // boundaries and the constant-rate counter at both ends, behind the window partials
+  // (the caller makes the workspace 64 bytes per unit larger).
+  long long stamp[8];
+  int nstamp = 0;
+  const long long wall0 = wall_clock64();
+#define ZP_STAMP() do { stamp[nstamp++] = clock64(); } while (0)
+#else
+#define ZP_STAMP() do { } while (0)
+#endif
+  ZP_STAMP();
   // unit -> (item, row block): workgroup ids are dealt round-robin to the 8 XCDs; the row blocks
   // of an item get consecutive ids ON ONE XCD, so they run at the same time behind one L2 and
   // the item's keys leave HBM once
@@ -851,32 +861,35 @@ __global__ __launch_bounds__(kThreads, 2) void score_resident_kernel(ScoreArgs p
   const int l = item / (p.Hkv * p.B);
   const int Tn = p.NB * p.BS;
 
-  if (wave == 0) {
-    const int code = lane < p.NB ? p.table[(int64_t)b * p.NB + lane] : -1;
+  // Every wave builds the list of usable pages for itself (no LDS, no barrier): lane j reads table
+  // entry j, a ballot ranks the usable ones, and a lane permute leaves entry n of the list in lane
+  // n as (page id, table index | last << 30).
+  const int code = lane < p.NB ? p.table[(int64_t)b * p.NB + lane] : -1;
+  int seq = p.seq_idx[b];
+  int2 myinfo;
+  int nvalid;
+  {
     const int pid = page_is_pad(code) ? -1 : page_id(code);
     const bool ok = pid >= 0 && pid < p.num_pages;
     const unsigned long long okm = __builtin_amdgcn_ballot_w64(ok);
-    if (ok) {
-      const int n = __builtin_popcountll(okm & lanemask_lt());
-      vinfo[n] = make_int2(pid, lane | (page_is_last(code) ? (1 << 30) : 0));
-    }
-    if (lane == 0) nvalid_s = __builtin_popcountll(okm);
+    nvalid = __builtin_popcountll(okm);
+    const int dst = ok ? __builtin_popcountll(okm & lanemask_lt())
+                       : nvalid + __builtin_popcountll(~okm & lanemask_lt());
+    myinfo.x = __builtin_amdgcn_ds_permute(dst << 2, pid);
+    myinfo.y = __builtin_amdgcn_ds_permute(dst << 2, lane | (page_is_last(code) ? (1 << 30) : 0));
   }
   const int dpieces = p.D * T::bytes / 16;
   char* kb = smem + wave * 2 * kSubBytes;    // this wave's two K blocks
-  if (dpieces < 16)   // the tail of every staged row must read as zero
+  if (dpieces < 16) {   // the tail of every staged row must read as zero
     for (int i = lane; i < 2 * kSubBytes / 4; i += 64) ((uint32_t*)kb)[i] = 0u;
-  __syncthreads();
-  const int nvalid = nvalid_s;
-  // lane j keeps entry j of the valid-page list: (page id, table index | last << 30)
-  const int2 myinfo = lane < nvalid ? vinfo[lane] : make_int2(0, 0);
-  int seq = p.seq_idx[b];
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
   const bool seq_ok = seq >= 0 && seq < p.max_seqs;
   if (!seq_ok) seq = 0;
 
   const int tiles_per_page = TPP > 0 ? TPP : p.BS / 128;
   const int ntiles = nvalid * tiles_per_page;
-  auto tile_page = [&](int tile) { return TPP > 0 ? tile / TPP : tile / tiles_per_page; };
+  auto tile_page = [&](int tile) { return tile / (TPP > 0 ? TPP : tiles_per_page); };
   auto page_word = [&](int v, int vp) {   // entry vp of the list, wave-uniform
     if constexpr (TPP > 0) return __builtin_amdgcn_readlane(v, vp);
     else return __builtin_amdgcn_readfirstlane(__builtin_amdgcn_ds_bpermute(vp << 2, v));
@@ -901,8 +914,13 @@ __global__ __launch_bounds__(kThreads, 2) void score_resident_kernel(ScoreArgs p
     const __amdgpu_buffer_rsrc_t rs =
         __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, (int)(32 * k_row), 0x00020000);
     if (st_ok) {
+#ifdef ZP_RES_HALFDMA   // measurement only: half of the rows are fetched, results are wrong
+#define ZP_DMA_N 4
+#else
+#define ZP_DMA_N 8
+#endif
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
+      for (int i = 0; i < ZP_DMA_N; ++i)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lptr_t)(buf + i * kGrp), 16, st_off,
                                                  i * grp_step, 0, 0);
     }
@@ -934,37 +952,52 @@ __global__ __launch_bounds__(kThreads, 2) void score_resident_kernel(ScoreArgs p
 #pragma unroll
   for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(afrag[s]));
 
+  ZP_STAMP();
   const int row0 = rb * 32 + half * 4;   // rows of this lane: row0 + (r/4)*8 + r%4
   uint32_t lg[kResTiles * 8];
   float run[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r) run[r] = -INFINITY;
 
-  // ---- the sweep: products, causal mask, running maximum, rounded logits into registers
+  // ---- the sweep: products, causal mask, running maximum, rounded logits into registers.
+  // Software-pipelined inside the wave: the products of block it+1 are issued before the
+  // vector work on block it, so the matrix core runs under it.
+  auto products = [&](int it) {
+    const char* cur = kb + (it & 1) * kSubBytes + rd_off;
+    f32x16_t acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+    for (int s0 = 0; s0 < KS; s0 += 4) {
+      Frag bfr[4];
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+        bfr[s] = *(const Frag*)(cur + ((s0 + s) >> 1) * 256 + ((s0 + s) & 1) * 32);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) acc = M::mma(afrag[s0 + s], bfr[s], acc);
+    }
+    return acc;
+  };
+  f32x16_t acc_cur;
+  if (ntiles > 0) acc_cur = products(0);
+  // every fragment of block 0 is in registers: block 2 may overwrite it
+  asm volatile("" ::: "memory");
+  if (ntiles > 2) issue(2, kb);
 #pragma unroll
   for (int it = 0; it < kResTiles; ++it) {
     if (it < ntiles) {
-      // block `it` has landed once at most the 8 loads of block it+1 are outstanding
-      if (it >= 2) {
-        if (it + 1 < ntiles) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      f32x16_t acc_next;
+      if (it + 1 < ntiles) {
+        // block it+1 has landed once at most the 8 loads of block it+2 are outstanding
+        if (it + 1 >= 2) {
+          if (it + 2 < ntiles) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(ZP_DMA_N) : "memory");
+          else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        acc_next = products(it + 1);
+        asm volatile("" ::: "memory");
+        if (it + 3 < ntiles) issue(it + 3, kb + ((it + 1) & 1) * kSubBytes);
       }
-      const char* cur = kb + (it & 1) * kSubBytes + rd_off;
-      f32x16_t acc;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-#pragma unroll
-      for (int s0 = 0; s0 < KS; s0 += 4) {
-        Frag bfr[4];
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
-          bfr[s] = *(const Frag*)(cur + ((s0 + s) >> 1) * 256 + ((s0 + s) & 1) * 32);
-#pragma unroll
-        for (int s = 0; s < 4; ++s) acc = M::mma(afrag[s0 + s], bfr[s], acc);
-      }
-      // every fragment of this buffer is in registers: block it+2 may overwrite it
-      asm volatile("" ::: "memory");
-      if (it + 2 < ntiles) issue(it + 2, kb + (it & 1) * kSubBytes);
+      f32x16_t acc = acc_cur;
       const int vp = tile_page(it);
       const int vs = page_word(myinfo.y, vp);
       const int toff = (it - vp * tiles_per_page) * 128 + wtok;
@@ -981,9 +1014,11 @@ __global__ __launch_bounds__(kThreads, 2) void score_resident_kernel(ScoreArgs p
 #pragma unroll
       for (int r = 0; r < 16; r += 2)
         lg[it * 8 + (r >> 1)] = P2::pack(acc[r] * p.scale, acc[r + 1] * p.scale);
+      if (it + 1 < ntiles) acc_cur = acc_next;
     }
   }
 
+  ZP_STAMP();
   // ---- row maximum over the lanes of a row and the four waves
   auto row_slot = [&](int r) { return (r >> 2) * 8 + half * 4 + (r & 3); };
   float mx[16];
@@ -1003,6 +1038,7 @@ __global__ __launch_bounds__(kThreads, 2) void score_resident_kernel(ScoreArgs p
   }
   __syncthreads();
 
+  ZP_STAMP();
   // ---- x = rounded(logit - max) back into the registers, row sums of exp(x)
 #pragma unroll
   for (int r = 0; r < 16; ++r) run[r] = 0.f;
@@ -1019,6 +1055,7 @@ __global__ __launch_bounds__(kThreads, 2) void score_resident_kernel(ScoreArgs p
       }
     }
   }
+  ZP_STAMP();
   float cl[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
@@ -1038,6 +1075,7 @@ __global__ __launch_bounds__(kThreads, 2) void score_resident_kernel(ScoreArgs p
     cl[r] = ok ? -__builtin_amdgcn_logf(v) : -INFINITY;   // rows outside the window or group never win a maximum
   }
 
+  ZP_STAMP();
   // ---- output: p = 2^(x log2(e) - log2(sum)), group maximum, this block's share of the window sum
   float* part = p.part + ((int64_t)item * p.RB + rb) * Tn + wtok + col;
 #pragma unroll
@@ -1057,6 +1095,15 @@ __global__ __launch_bounds__(kThreads, 2) void score_resident_kernel(ScoreArgs p
       if (half == 0) __builtin_nontemporal_store(red, part + j * p.BS + toff);
     }
   }
+  ZP_STAMP();
+#ifdef ZP_RES_STAMP
+  if (tid == 0) {
+    long long* dst = (long long*)(p.part + (int64_t)p.n_items * p.RB * Tn) + (int64_t)(item * p.RB + rb) * 8;
+    for (int i = 0; i < 7; ++i) dst[i] = stamp[i];
+    dst[7] = wall_clock64() - wall0;
+  }
+#endif
+#undef ZP_STAMP
 }
 
 // Adds the row blocks' window partials of every (layer, sequence, head) in block order, divides by
@@ -1067,24 +1114,44 @@ __global__ __launch_bounds__(256) void score_combine_kernel(const float* __restr
                                                             const int32_t* __restrict__ table,
                                                             int B, int NB, int BS, int Hkv, int RB,
                                                             int W, int num_pages, int rmax) {
+  // four consecutive tokens per thread (a page is a multiple of 128 tokens)
   const int item = blockIdx.x;
   const int b = (item / Hkv) % B;
   const int Tn = NB * BS;
-  const int t = blockIdx.y * 256 + threadIdx.x;
+  const int t = (blockIdx.y * 256 + threadIdx.x) * 4;
   if (t >= Tn) return;
   const int code = table[(int64_t)b * NB + t / BS];
   const int pid = page_is_pad(code) ? -1 : page_id(code);
-  float v = 0.f;
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  f4 v = {0.f, 0.f, 0.f, 0.f};
   if (pid >= 0 && pid < num_pages) {
     const float* src = part + (int64_t)item * RB * Tn + t;
-    v = __builtin_nontemporal_load(src);
+    v = __builtin_nontemporal_load((const f4*)src);
     for (int r = 1; r < RB; ++r) {
-      const float o = __builtin_nontemporal_load(src + (int64_t)r * Tn);
-      v = rmax ? fmaxf(v, o) : v + o;
+      const f4 o = __builtin_nontemporal_load((const f4*)(src + (int64_t)r * Tn));
+      if (rmax) { v.x = fmaxf(v.x, o.x); v.y = fmaxf(v.y, o.y); v.z = fmaxf(v.z, o.z); v.w = fmaxf(v.w, o.w); }
+      else { v.x += o.x; v.y += o.y; v.z += o.z; v.w += o.w; }
     }
-    if (!rmax) v = Elem<T>::rnd(v / (float)W);
+    if (!rmax) {
+      v.x = Elem<T>::rnd(v.x / (float)W); v.y = Elem<T>::rnd(v.y / (float)W);
+      v.z = Elem<T>::rnd(v.z / (float)W); v.w = Elem<T>::rnd(v.w / (float)W);
+    }
   }
-  Elem<T>::st(out, (int64_t)item * Tn + t, v);
+  const int64_t o = (int64_t)item * Tn + t;
+  if constexpr (T::bytes == 2) {
+    uint16_t* dst = (uint16_t*)out + o;
+    if constexpr (std::is_same<T, BF16>::value) {
+      const uint2 w = make_uint2(float_to_bf16_bits(v.x) | ((uint32_t)float_to_bf16_bits(v.y) << 16),
+                                 float_to_bf16_bits(v.z) | ((uint32_t)float_to_bf16_bits(v.w) << 16));
+      *(uint2*)dst = w;
+    } else {
+      const uint2 w = make_uint2(float_to_f16_bits(v.x) | ((uint32_t)float_to_f16_bits(v.y) << 16),
+                                 float_to_f16_bits(v.z) | ((uint32_t)float_to_f16_bits(v.w) << 16));
+      *(uint2*)dst = w;
+    }
+  } else {
+    *(f4*)((float*)out + o) = v;
+  }
 }
 
 }  // namespace
@@ -1196,9 +1263,9 @@ extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
   a.n_items = L * B * Hkv;
   a.part = (float*)workspace;
   if (resident) {
-    const size_t smem = (size_t)kWaves * 2 * kSubBytes + sizeof(float) * kWaves * 32 + sizeof(int2) * NB;
+    const size_t smem = (size_t)kWaves * 2 * kSubBytes + sizeof(float) * kWaves * 32;
     const unsigned units = (unsigned)(((int64_t)a.n_items + 7) / 8 * 8 * RB);
-    const dim3 cgrid((unsigned)a.n_items, (unsigned)((NB * BS + 255) / 256));
+    const dim3 cgrid((unsigned)a.n_items, (unsigned)((NB * BS / 4 + 255) / 256));
 #define ZP_RESIDENT_LAUNCH(TT)                                                                   \
   do {                                                                                           \
     void (*fn)(ScoreArgs) = score_resident_kernel<TT, 0, -1, 0>;                                 \
