@@ -316,11 +316,21 @@ def _score_three_sweeps(k, q, seq_idx, enc, reduced="mean"):
     B, NB = enc.shape
     lib = _lib.load()
     out = torch.empty((L, B, Hkv, NB, BS), device=k.device, dtype=k.dtype)
-    assert lib.zp_attention_score_workspace(L, B, NB, BS, Hkv, Hq, W) > 0
+    full = lib.zp_attention_score_workspace(L, B, NB, BS, Hkv, Hq, W)
+    assert full > 0
+    # more than 128 window x group rows: the three-sweep kernel keeps fp32 partial sums of its
+    # own (one row of the scores), still less than the one-sweep kernel asks for
+    gp = 1
+    while gp < Hq // Hkv:
+        gp *= 2
+    floor = L * B * Hkv * NB * BS * 4 if (W * gp + 31) // 32 > 4 else 0
+    assert floor < full
+    ws = torch.empty(max(floor, 1), device=k.device, dtype=torch.uint8)
     _lib.call("zp_attention_score", _lib.dev_ptr(k), _lib.dev_ptr(q), _lib.dev_ptr(seq_idx),
               _lib.dev_ptr(enc), _lib.dev_ptr(out), 0, L, B, NB, BS, Hkv, Hq, D, W, P, S,
               k.stride(0), k.stride(1), q.stride(0), q.stride(1), float(D ** -0.5),
-              {"mean": 0, "max": 1}[reduced], _lib.dtype_tag(k), 0, 0, _lib.stream_ptr(k))
+              {"mean": 0, "max": 1}[reduced], _lib.dtype_tag(k), _lib.dev_ptr(ws) if floor else 0,
+              floor, _lib.stream_ptr(k))
     return out
 
 
