@@ -6,8 +6,10 @@ top-2048 per kv head -> in-place compaction to 8 pages) over one batch of synthe
 sequences at Qwen3-8B attention shape (32 q heads, 8 kv heads, head_dim 128, bf16, page 256,
 window 32), inputs resident in HBM.  The default workload is the one the metric is quoted on,
 BASELINE configs[3]: 256 ragged sequences of 9-10 pages, groups of 16 sharing two prefix pages
-(copy-on-write targets), all 36 layers per step (one layer at a time over one page pool).
-Prints ONE JSON line.
+(copy-on-write targets), all 36 layers per step, one layer per call.  The cache is ONE allocation
+(2, 4, 60000 pages, 256, 8, 128) with K and V as its halves -- the way the engine and the reference
+allocate theirs -- and the 36 layers take its four layer slices in turn, so that no layer finds the
+previous layer's pages in a cache.  Prints ONE JSON line.
 
 After it, unless --no-extra-legs, the same process adds the 64-sequence single-layer workload
 (BASELINE configs[1]) as `configs1_b64`, and, unless --no-e2e, BASELINE's end-to-end case
@@ -49,9 +51,9 @@ def cpu_baseline(wl, cfg, sample_seqs, layers=1, budget_s=30.0):
     from oracle import zipage_oracle as O
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    from zipage_amd.workload import cpu_subset
+    from zipage_amd.bench.workload import cpu_subset
     b = min(sample_seqs, wl.B)
-    sub = cpu_subset(wl, range(b))
+    sub = cpu_subset(wl, range(b), layer=0)
     k, v, q = sub["k"], sub["v"], sub["q"]
     enc, tgt, comp, qid = sub["block_tables"], sub["targets"], sub["compressed"], sub["query_ids"]
     times = []
@@ -150,7 +152,7 @@ def run_pipeline(config, args, sw="pooling", batch=None, steps=None, warmup=None
     stage.  Returns the JSON-ready dict of the run (without the contract's fixed keys)."""
     import torch
     from zipage_amd.compress import CompressConfig, StageTimer, compress_layers
-    from zipage_amd.workload import algorithmic_bytes, ragged_batch
+    from zipage_amd.bench.workload import algorithmic_bytes, ragged_batch
 
     steps = args.steps if steps is None else steps
     warmup = args.warmup if warmup is None else warmup
@@ -159,16 +161,17 @@ def run_pipeline(config, args, sw="pooling", batch=None, steps=None, warmup=None
         wl = ragged_batch(batch, L=1, pool_pages=20000, budget=8, W=16 if sw == "scripts" else 32,
                           seed=1, lengths=(2049, 2304), name="cfg2",
                           with_score_cache=sw == "scripts", compressed=sw == "scripts",
-                          place_tries=args.place_tries)
+                          place_tries=args.place_tries, one_allocation=args.place_tries <= 1)
         desc = (f"configs[1]: {batch} ragged sequences, 1 layer, Qwen3-8B attention shape (32q/8kv "
                 "heads, head_dim 128), bf16, 9 pages x 256 tokens, window 32, 20k-page pool, score "
                 "-> max-pool 7 -> top-2048/head -> compact to 8 pages")
     elif config == 3:
-        from zipage_amd.workload import QWEN3_0_6B
+        from zipage_amd.bench.workload import QWEN3_0_6B
         batch, layers = batch or 128, 1
         wl = ragged_batch(batch, L=1, pool_pages=2048, budget=8, W=32, seed=0, lengths=(2304, 2304),
                           dtype=torch.float32, shape=QWEN3_0_6B, name="cfg3", with_score_cache=True,
-                          compressed=True, place_tries=args.place_tries)
+                          compressed=True, place_tries=args.place_tries,
+                          one_allocation=args.place_tries <= 1)
         desc = (f"configs[2]: {batch} sequences, 1 layer, Qwen3-0.6B attention shape (16q/8kv heads, "
                 "head_dim 128), fp32, 9 pages x 256 tokens, window 32, 2048-page pool, score -> global "
                 "score (U(0,1) carried, decay 0.9, added) -> avg-pool 7 -> minus 0.5 x "
@@ -176,14 +179,27 @@ def run_pipeline(config, args, sw="pooling", batch=None, steps=None, warmup=None
                 + " redundancy (lambda 2/3) -> top-2048/head -> compact to 8 pages")
     else:
         batch, layers = batch or 256, 36
-        wl = ragged_batch(batch, L=1, pool_pages=60000, budget=8, W=32, seed=3,
-                          lengths=(2049, 2560), shared_prefix_group=16, shared_prefix_pages=2,
-                          name="cfg4", place_tries=args.place_tries)
+        # ONE cache tensor (2, slices, 60000 pages, ...), K and V its two halves, as the engine and
+        # the reference allocate theirs; the 36 layers of a step take its layer slices in turn, so
+        # no launch finds the previous layer's pages in a cache.  Placed pools (--place-tries > 1)
+        # are separate allocations and an extra report, never the headline.
+        wl, pool_slices = None, args.pool_slices
+        while wl is None:
+            try:
+                wl = ragged_batch(batch, L=pool_slices, pool_pages=60000, budget=8, W=32, seed=3,
+                                  lengths=(2049, 2560), shared_prefix_group=16, shared_prefix_pages=2,
+                                  name="cfg4", one_allocation=True)
+            except torch.cuda.OutOfMemoryError:
+                if pool_slices == 1:
+                    raise
+                pool_slices //= 2
+                torch.cuda.empty_cache()
         desc = (f"configs[3]: {batch} ragged sequences (9-10 pages x 256 tokens), groups of 16 share "
-                "2 prefix pages (copy-on-write targets), 60k-page pool, Qwen3-8B attention shape "
-                "(32q/8kv heads, head_dim 128), bf16, window 32, score -> max-pool 7 -> "
-                "top-2048/head -> compact to 8 pages, 36 layers per step run one layer at a time "
-                "over the same pool")
+                "2 prefix pages (copy-on-write targets), Qwen3-8B attention shape (32q/8kv heads, "
+                "head_dim 128), bf16, window 32, score -> max-pool 7 -> top-2048/head -> compact to 8 "
+                f"pages; one cache allocation (2, {pool_slices}, 60000 pages, 256, 8, 128) = "
+                f"{2 * pool_slices * 60000 * 524288 / 1e9:.0f} GB with K and V as its halves; a step "
+                f"is 36 layers, one layer per call, over the {pool_slices} layer slices in turn")
     cfg = CompressConfig(budget_blocks=8, query_cache_len=32, enable_pooling=True, pooling_size=7)
     if config == 3:
         if sw == "scripts":
@@ -207,10 +223,16 @@ def run_pipeline(config, args, sw="pooling", batch=None, steps=None, warmup=None
                                  lightning_redudancy=False, enable_pooling=True, pooling_size=7)
             desc += " [NOT the headline switches: raw all-pairs redundancy added]"
 
+    slices = wl.L if layers > 1 else 1
+    sc = wl.score_cache
+
     def step(timer=None):
-        for _ in range(layers):
-            compress_layers(wl.k, wl.v, wl.q, wl.score_cache, wl.query_ids, wl.block_tables,
-                            wl.compressed, wl.targets, cfg, timer=timer,
+        for i in range(layers):
+            l = i % slices
+            compress_layers(wl.k[l:l + 1] if layers > 1 else wl.k, wl.v[l:l + 1] if layers > 1 else wl.v,
+                            wl.q[l:l + 1] if layers > 1 else wl.q,
+                            sc if sc is None or layers == 1 else sc[l:l + 1], wl.query_ids,
+                            wl.block_tables, wl.compressed, wl.targets, cfg, timer=timer,
                             fused_select=not args.separate_select_stages)
 
     for _ in range(warmup):
@@ -234,17 +256,18 @@ def run_pipeline(config, args, sw="pooling", batch=None, steps=None, warmup=None
     stage_s = timer.seconds()
     ms_per_step = elapsed / steps * 1e3
     seqs_per_s = wl.B / (elapsed / steps)
-    alg = algorithmic_bytes(wl, cfg)  # one layer
+    alg = algorithmic_bytes(wl, cfg, layers=1)  # one layer
     kv_s = kv_timer.seconds()["compress_kv"] / (steps * layers)
     achieved = alg["compress_kv"] / kv_s / 1e9
     stages_ms = {k: round(v / (stage_steps * layers) * 1e3, 4) for k, v in stage_s.items()}
     gpu_ms = sum(stage_s.values()) / (stage_steps * layers) * 1e3  # per layer
     if args.traffic is not None:
         traffic, traffic_src = args.traffic, "--traffic"
-    elif (config, wl.B) in COMPACT_TRAFFIC and sw == "pooling":
+    elif (config, wl.B) in COMPACT_TRAFFIC and sw == "pooling" and wl.placement is None:
         traffic, traffic_src = COMPACT_TRAFFIC[(config, wl.B)]
-        traffic_src = ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run of this workload, "
-                       "scaled by the calibration copy: " + traffic_src)
+        traffic_src = ("rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE per compact_kernel dispatch of this "
+                       "command in a counter run (counters cannot be read from inside a timed "
+                       "run), scaled by the calibration copy: " + traffic_src)
     else:
         traffic, traffic_src = None, "no counter run of this workload"
     roof = {"bound": "hbm", "kernel": "compact_kernel (compress_kv)",
@@ -252,7 +275,17 @@ def run_pipeline(config, args, sw="pooling", batch=None, steps=None, warmup=None
             "frac": round(achieved / HBM_PEAK_GBS, 4),
             "traffic": traffic, "traffic_source": traffic_src,
             "algorithmic_bytes": alg["compress_kv"],
-            "avg_launch_us": round(kv_s * 1e6, 2)}
+            "avg_launch_us": round(kv_s * 1e6, 2),
+            "pools": ("K and V are the halves of one cache allocation, as the engine allocates"
+                      if wl.placement is None else
+                      "K and V are separate allocations picked by a timed probe (bench only)")}
+    if slices > 1:
+        # the launches of the timed steps by the layer slice they worked on: where a slice's K
+        # and V lie in device memory moves this kernel by up to 15 %
+        per = [[] for _ in range(slices)]
+        for i, (_, st, ed) in enumerate(kv_timer.spans):
+            per[(i % layers) % slices].append(st.elapsed_time(ed) * 1e3)
+        roof["avg_launch_us_by_layer_slice"] = [round(sum(p) / len(p), 1) for p in per]
     out = {
         "value": round(seqs_per_s, 1),
         "unit": "sequences/s (one layer)" if layers == 1 else f"sequences/s ({layers} layers)",
@@ -325,14 +358,17 @@ def main():
     ap.add_argument("--separate-select-stages", action="store_true",
                     help="run pooling, the mask epilogue and top-k as three launches (timed under "
                          "the reference's stage names) instead of the one-launch selection")
-    ap.add_argument("--place-tries", type=int, default=16,
-                    help="most pool-sized allocations made side by side before any data is written "
-                         "(allocation stops as soon as a pair is fast or 160 GB are held); a timed "
-                         "compaction on pairs of them picks the K pool and the V pool (the "
+    ap.add_argument("--pool-slices", type=int, default=4,
+                    help="layer slices of the headline workload's cache allocation "
+                         "(2 x slices x 60000 pages x 512 KB; halved until it fits)")
+    ap.add_argument("--place-tries", type=int, default=1,
+                    help="--config 2 / 3 only, not the headline: above 1, K and V are separate "
+                         "allocations chosen among that many pool-sized ones made side by side "
+                         "before any data is written, by a timed compaction on pairs of them (the "
                          "in-place compaction is ~15 %% faster when the two lie in different regions "
-                         "of device memory); every probe figure is reported in 'placement' and the "
-                         "first-two-allocations figure in 'roofline'; 1 = take the first two "
-                         "allocations")
+                         "of device memory); every probe figure is reported in 'placement'.  1 "
+                         "(default) = one cache allocation with K and V as its halves, as the "
+                         "engine allocates")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-sample", type=int, default=64)
     ap.add_argument("--calibrate-copy", action="store_true",

@@ -25,13 +25,14 @@ def test_help_lists_the_contract_flags():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("extra", [["--config", "4"], ["--config", "2"], ["--config", "3"],
+@pytest.mark.parametrize("extra", [["--config", "4", "--pool-slices", "2"], ["--config", "2"],
+                                   ["--config", "3"], ["--config", "2", "--place-tries", "2"],
                                    ["--config", "2", "--pipeline-switches", "scripts"]])
 def test_bench_line_on_a_small_batch(extra):
     """One JSON line with the contract's keys, on a batch small enough for a test."""
     import json
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--batch", "4", "--steps", "2",
-                        "--warmup", "1", "--no-e2e", "--cpu-sample", "2", "--place-tries", "2", *extra],
+                        "--warmup", "1", "--no-e2e", "--cpu-sample", "2", *extra],
                        capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr[-2000:]
     lines = [l for l in r.stdout.splitlines() if l.startswith("{")]
@@ -46,10 +47,14 @@ def test_bench_line_on_a_small_batch(extra):
     assert roof["bound"] == "hbm" and roof["unit"] == "GB/s" and roof["peak"] == 8000.0
     assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
     assert out["cpu_baseline"]["kind"] == "port" and out["cpu_baseline"]["value"] > 0
-    assert out["placement"]["slabs"] == 2
-    first = roof["first_two_allocations"]
-    assert abs(first["frac"] - first["achieved"] / roof["peak"]) < 1e-3
     assert "traffic" in roof and "traffic_source" in roof
-    if extra == ["--config", "4"]:
+    if "--place-tries" in extra:   # separate pools picked by the probe: an extra report
+        assert out["placement"]["slabs"] == 2 and "separate allocations" in roof["pools"]
+        first = roof["first_two_allocations"]
+        assert abs(first["frac"] - first["achieved"] / roof["peak"]) < 1e-3
+    else:                          # the default: one cache allocation, as the engine makes it
+        assert "placement" not in out and "one cache allocation" in roof["pools"]
+    if extra[:2] == ["--config", "4"]:
         assert out["config"]["layers"] == 36 and "36 layers" in out["unit"]
+        assert len(roof["avg_launch_us_by_layer_slice"]) == 2
     assert "workload" in out["config"] and "model" not in out["config"]

@@ -102,7 +102,7 @@ def _oracle_sample(wl, sub, cfg_kwargs, seq_ids, scores_gpu, dtype):
 def test_config2_64_ragged_sequences(dev):
     """BASELINE configs[1]: 64 sequences, Qwen3-8B shape, bf16, 20k-page pool."""
     from zipage_amd.compress import CompressConfig
-    from zipage_amd.workload import cpu_subset, ragged_batch
+    from zipage_amd.bench.workload import cpu_subset, ragged_batch
     wl = ragged_batch(64, L=1, pool_pages=20000, budget=BUDGET, W=32, seed=1, lengths=(2049, 2304))
     kb, vb = _save_touched(wl)
     sub = cpu_subset(wl, [0, 17, 63])
@@ -128,7 +128,7 @@ def test_config4_prefix_sharing_copy_on_write(dev):
     lengths up to 2560 (9 or 10 pages), 60k-page pool; targets follow the copy-on-write rule so
     shared pages are read-only sources."""
     from zipage_amd.compress import CompressConfig
-    from zipage_amd.workload import cpu_subset, ragged_batch
+    from zipage_amd.bench.workload import cpu_subset, ragged_batch
     wl = ragged_batch(256, L=1, pool_pages=60000, budget=BUDGET, W=32, seed=3, lengths=(2049, 2560),
                       shared_prefix_group=16, shared_prefix_pages=2)
     assert wl.block_tables.shape[1] == 10 and (wl.block_tables == -1).any()
@@ -148,7 +148,7 @@ def test_config4_layer_chunk_of_four(dev):
     runner's `layer_stride` loop, zipage/engine/model_runner.py:466-469): the grid spans layers,
     every layer has its own keys, queries and flags, and every layer's compaction is checked."""
     from zipage_amd.compress import CompressConfig
-    from zipage_amd.workload import cpu_subset, ragged_batch
+    from zipage_amd.bench.workload import cpu_subset, ragged_batch
     wl = ragged_batch(256, L=4, pool_pages=6000, budget=BUDGET, W=32, seed=3, lengths=(2049, 2560),
                       shared_prefix_group=16, shared_prefix_pages=2)
     shared = sorted({t[0] for t in wl.tables} | {t[1] for t in wl.tables})
@@ -167,7 +167,7 @@ def test_config4_36_layers_in_chunks_of_eight(dev):
     ragged sequences with shared prefix pages.  Every layer is checked for the stable in-place
     gather; three layers of two sequences are compared with the oracle end to end."""
     from zipage_amd.compress import CompressConfig, compress_layers
-    from zipage_amd.workload import cpu_subset, ragged_batch
+    from zipage_amd.bench.workload import cpu_subset, ragged_batch
     L, stride = 36, 8
     wl = ragged_batch(32, L=L, pool_pages=400, budget=BUDGET, W=32, seed=9, lengths=(2049, 2560),
                       shared_prefix_group=16, shared_prefix_pages=2)
@@ -203,7 +203,7 @@ def test_config1_single_sequence_fp32_full_oracle(dev):
     """BASELINE configs[0]: one sequence, Qwen3-0.6B shape (16 q / 8 kv heads), fp32, 9 pages
     from a 64-page pool, window 32, max-pool 7, keep 2048 -- compared in full with the oracle."""
     from zipage_amd.compress import CompressConfig
-    from zipage_amd.workload import QWEN3_0_6B, cpu_subset, ragged_batch
+    from zipage_amd.bench.workload import QWEN3_0_6B, cpu_subset, ragged_batch
     wl = ragged_batch(1, L=1, pool_pages=64, budget=BUDGET, W=32, seed=0, lengths=(2304, 2304),
                       dtype=torch.float32, shape=QWEN3_0_6B)
     sub = cpu_subset(wl, [0])
@@ -233,7 +233,7 @@ def test_config3_global_score_and_redundancy_128_sequences(dev, variant):
     redundancy (lambda 2/3), lightning or all-pairs redundancy; properties on the whole batch,
     the oracle's full pipeline on two of the sequences."""
     from zipage_amd.compress import CompressConfig
-    from zipage_amd.workload import QWEN3_0_6B, cpu_subset, ragged_batch
+    from zipage_amd.bench.workload import QWEN3_0_6B, cpu_subset, ragged_batch
     wl = ragged_batch(128, L=1, pool_pages=2048, budget=BUDGET, W=32, seed=0, lengths=(2304, 2304),
                       dtype=torch.float32, shape=QWEN3_0_6B, with_score_cache=True, compressed=True)
     kb, vb = _save_touched(wl)

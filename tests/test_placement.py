@@ -2,7 +2,7 @@
 import pytest
 import torch
 
-from zipage_amd.placement import place_kv_pools, place_pools
+from zipage_amd.bench.placement import place_kv_pools, place_pools
 
 
 def test_place_pools_keeps_fastest_and_releases_the_rest():
@@ -83,7 +83,7 @@ def test_place_kv_pools_limits():
 @pytest.mark.gpu
 def test_placed_workload_runs_the_pipeline():
     from zipage_amd.compress import CompressConfig, compress_layers
-    from zipage_amd.workload import ragged_batch
+    from zipage_amd.bench.workload import ragged_batch
     wl = ragged_batch(4, L=1, pool_pages=64, budget=8, W=32, seed=5, lengths=(2049, 2304),
                       place_tries=2)
     assert wl.placement["slabs"] == 2 and set(wl.placement["probe_us"]) == {"0-1"}

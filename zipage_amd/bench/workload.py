@@ -50,14 +50,16 @@ def encode_tables(tables, device):
 def ragged_batch(B, *, L=1, pool_pages=20000, budget=8, W=32, BS=256, dtype=torch.bfloat16,
                  seed=1, lengths=(2049, 2304), shared_prefix_group=0, shared_prefix_pages=2,
                  with_score_cache=False, compressed=False, shape=QWEN3_8B, device="cuda:0",
-                 name="ragged", place_tries=1):
+                 name="ragged", place_tries=1, one_allocation=False):
     """B sequences with token counts uniform in ``lengths`` (rounded up to whole pages, since
     compression fires only on a full last page), pages drawn without replacement from a pool
     of ``pool_pages`` ids.  With ``shared_prefix_group = n`` every group of n sequences shares
     its first ``shared_prefix_pages`` pages (copy-on-write targets).  With ``place_tries > 1``
     the K and V pools are chosen by ``placement.place_kv_pools`` among that many pool-sized
     allocations made side by side (a timed gather on pairs of them, before any data is
-    written); the report is kept in ``placement``."""
+    written); the report is kept in ``placement``.  With ``one_allocation`` K and V are the two
+    halves of ONE ``(2, L, pool_pages, BS, Hkv, D)`` tensor, which is how the engine and the
+    reference allocate their cache (zipage/engine/model_runner.py:219-307)."""
     g = torch.Generator().manual_seed(seed)
     Hq, Hkv, D = shape["Hq"], shape["Hkv"], shape["D"]
     lens = torch.randint(lengths[0], lengths[1] + 1, (B,), generator=g)
@@ -98,8 +100,11 @@ def ragged_batch(B, *, L=1, pool_pages=20000, budget=8, W=32, BS=256, dtype=torc
         return torch.empty((L, pool_pages, BS, Hkv, D), dtype=dtype, device=dev)
 
     placement = None
-    if place_tries > 1:
-        from zipage_amd.placement import place_kv_pools, probe_gather_us
+    if one_allocation:
+        kv = torch.empty((2, L, pool_pages, BS, Hkv, D), dtype=dtype, device=dev)
+        k, v = kv[0], kv[1]
+    elif place_tries > 1:
+        from zipage_amd.bench.placement import place_kv_pools, probe_gather_us
         (k, v), placement = place_kv_pools(
             alloc_one, lambda kp, vp: probe_gather_us(kp, vp, block_tables, compressed_t, targets_t,
                                                       budget * BS), place_tries,
@@ -126,11 +131,13 @@ def ragged_batch(B, *, L=1, pool_pages=20000, budget=8, W=32, BS=256, dtype=torc
         budget=budget, W=W, tables=tables, placement=placement)
 
 
-def algorithmic_bytes(wl: Workload, cfg) -> dict:
-    """HBM bytes each stage has to move for this workload (per launch over all layers):
+def algorithmic_bytes(wl: Workload, cfg, layers=None) -> dict:
+    """HBM bytes each stage has to move for this workload (per launch over ``layers`` layers, all
+    of the workload's by default):
     K once + Q + score out for the scorer; score-cache read+write for the global score;
     K and V survivors read+written for the compaction."""
     L, _, BS, Hkv, D = wl.k.shape
+    L = L if layers is None else layers
     Hq = wl.q.shape[3]
     es = wl.k.element_size()
     valid_pages = sum(len(t) for t in wl.tables)
@@ -150,11 +157,12 @@ def algorithmic_bytes(wl: Workload, cfg) -> dict:
     return out
 
 
-def cpu_subset(wl: Workload, seq_ids):
-    """Host copy of the sequences ``seq_ids`` with their pages renumbered densely, for checking
-    or timing against a CPU implementation.  Returns a dict of CPU tensors with the same
-    meaning as the Workload fields (block tables already encoded)."""
+def cpu_subset(wl: Workload, seq_ids, layer=None):
+    """Host copy of the sequences ``seq_ids`` (all layers, or the one given) with their pages
+    renumbered densely, for checking or timing against a CPU implementation.  Returns a dict of
+    CPU tensors with the same meaning as the Workload fields (block tables already encoded)."""
     seq_ids = list(seq_ids)
+    lsel = slice(None) if layer is None else slice(layer, layer + 1)   # a view, never a pool copy
     tables = [wl.tables[b] for b in seq_ids]
     targets = wl.targets[seq_ids].tolist()
     used = sorted({p for t in tables for p in t} | {int(p) for row in targets for p in row})
@@ -165,8 +173,8 @@ def cpu_subset(wl: Workload, seq_ids):
     enc = torch.tensor([r[:-1] + [-r[-1] - 2] + [-1] * (width - len(r)) for r in rows],
                        dtype=torch.int32)
     return dict(
-        k=wl.k[:, idx].cpu(), v=wl.v[:, idx].cpu(), q=wl.q[:, seq_ids].cpu(),
-        score_cache=None if wl.score_cache is None else wl.score_cache[:, idx].cpu(),
+        k=wl.k[lsel][:, idx].cpu(), v=wl.v[lsel][:, idx].cpu(), q=wl.q[lsel][:, seq_ids].cpu(),
+        score_cache=None if wl.score_cache is None else wl.score_cache[lsel][:, idx].cpu(),
         query_ids=torch.arange(len(seq_ids), dtype=torch.int32), block_tables=enc,
         compressed=wl.compressed[seq_ids].cpu(),
         targets=torch.tensor([[remap[int(p)] for p in row] for row in targets], dtype=torch.int32),
