@@ -59,7 +59,12 @@ int zp_store_query(const void* query, void* query_cache, const int32_t* slot_map
  * k_cache (L, num_pages, BS, Hkv, D), query_cache (L, max_seqs, W, Hq, D), both
  * contiguous in their last two axes; scores_out (L, B, Hkv, NB, BS) contiguous, in the
  * cache dtype; logits_out NULL or (L, B, Hq, W, NB, BS) contiguous.
- * workspace: zp_attention_score_workspace() bytes of device scratch. */
+ * workspace: zp_attention_score_workspace() bytes of device scratch -- an upper bound over
+ * the dtypes.  With 16-bit caches, no logits_out, a positive scale and at most 2560 tokens per
+ * sequence that scratch lets the library keep the rounded logits in registers and sweep K once
+ * (fp32 window partials per block of 32 query rows go through the scratch); with less scratch
+ * (NULL is fine up to 128 window x group rows) the same entry point sweeps K three times.  The
+ * two kernels round at the same points and differ only in the fp32 order of the row sums. */
 int zp_attention_score(const void* k_cache, const void* query_cache, const int32_t* seq_idx,
                        const int32_t* block_table, void* scores_out, void* logits_out,
                        int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
@@ -172,8 +177,11 @@ int zp_select_topk(const void* scores, void* scores_out, const void* redundancy,
  * zipage/kernel/compress_kv.py:103-141 (kernel :8-100).
  * key/value (L, num_pages, BS, Hkv, D) with the given element strides (head_dim stride
  * 1); flag (L, B, Hkv, NB, BS) bytes contiguous; target (B, target_width) int32.
- * Stable in-place compaction; a target page may alias a source page of the same
- * sequence at the same or a lower logical index. */
+ * Stable in-place compaction.  A target page may be one of the sequence's own source pages
+ * only if that source page sits at the same or a LATER position of block_table than the
+ * position the page has in target_block_table (source index >= target index: survivors only
+ * ever move towards the front), which is what BlockManager.may_compress produces
+ * (zipage/engine/block_manager.py:129-169). */
 int zp_compress_kv(void* key, void* value, const uint8_t* flag, const int32_t* block_table,
                    const int32_t* target_block_table, int32_t L, int32_t B, int32_t NB,
                    int32_t BS, int32_t Hkv, int32_t D, int32_t num_pages,
@@ -265,10 +273,16 @@ int zp_compress_layers(void* k_cache, void* v_cache, const void* query_cache, vo
  * hipMalloc / hipFree or allocating routine; flag_out may be NULL (the flags then live in the
  * array too).  A chunk whose zp_compress_layers_workspace() exceeds the array is refused with
  * ZP_EINVAL: 32 MiB covers one layer of 256 sequences x 10 pages at 8 kv heads in a 16-bit
- * dtype with the lightning redundancy on.  Every call on a GPU uses that GPU's one array: calls
- * that overlap in time on one GPU (two streams, two threads) race and must be serialised by the
- * caller.  Nothing in the array has to be cleared between calls. */
+ * dtype with the lightning redundancy on.  The array is too small for the scorer's window
+ * partials beyond ~90 such sequences per layer; larger chunks that still fit run the scorer's
+ * three-sweep kernel (same rounding points, see zp_attention_score).  Every call on a GPU uses
+ * that GPU's one array: calls that overlap in time on one GPU (two streams, two threads) race
+ * and must be serialised by the caller.  Nothing in the array has to be cleared between calls.
+ * zp_static_scratch_init() looks the array's address up for the current device (once per
+ * device; the entry point does it on its first call otherwise): a caller that captures the
+ * entry point into a HIP graph calls it beforehand, outside the capture. */
 #define ZP_STATIC_SCRATCH_BYTES (32u << 20)
+int zp_static_scratch_init(void);
 int zp_compress_layers_static(void* k_cache, void* v_cache, const void* query_cache,
                               void* score_cache, const int32_t* seq_idx,
                               const int32_t* block_table, const uint8_t* compressed,

@@ -511,7 +511,9 @@ def compress_pipeline(k_cache, v_cache, query_cache, score_cache, query_ids, blo
     compress_score.  Mutates ``k_cache``, ``v_cache`` and ``score_cache`` in place and
     returns the keep flag (and the final scores when asked).  ``deterministic_carry`` is this
     build's race-free handling of the score cache: ``global_score`` only reads it and the
-    carried scores of the survivors are compacted from the scores it returned."""
+    carried scores of the survivors are compacted from the scores it returned.  It is off by
+    default here (this function restates the reference) and on by default in the product's
+    ``compress_layers``: pass it explicitly to both when comparing them."""
     BS = k_cache.shape[2]
     scores = attention_score(k_cache, query_cache, query_ids, block_table, softmax_scale,
                              reduced, rounding=rounding)

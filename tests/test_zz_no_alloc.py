@@ -26,15 +26,16 @@ def _case(dev, dtype, seed, L, B, kw, budget=2, W=16, Hkv=2, Hq=8, nb=(3, 4)):
     return [t.to(dev) for t in (k, v, q, sc, qid, enc, comp, target)], cfg
 
 
-def _call(entry, tensors, cfg, flag_in_scratch=False):
-    """Runs `entry` on clones of the caches; returns (flag or None, k, v, score cache)."""
+def _call(entry, tensors, cfg, flag_in_scratch=False, deterministic_carry=True, check_memory=False):
+    """Runs `entry` on clones of the caches; returns (flag or None, k, v, score cache).  With
+    ``check_memory`` the free device memory is read right before and right after the call."""
     from zipage_amd import _lib
     from zipage_amd.compress import c_config, layer_chunk_args
     k, v, q, sc, qid, enc, comp, target = tensors
     k, v, sc = k.clone(), v.clone(), sc.clone()
     dims, strides = layer_chunk_args(k, v, q, sc, qid, enc, comp, target)
     L, B, NB, BS, Hkv, Hq, D, W = dims[:8]
-    cc = c_config(cfg)
+    cc = c_config(cfg, deterministic_carry=deterministic_carry)
     tag = _lib.dtype_tag(k)
     flag = None if flag_in_scratch else torch.zeros((L, B, Hkv, NB, BS), dtype=torch.bool, device=k.device)
     head = (k.data_ptr(), v.data_ptr(), q.data_ptr(), sc.data_ptr(), qid.data_ptr(), enc.data_ptr(),
@@ -42,7 +43,12 @@ def _call(entry, tensors, cfg, flag_in_scratch=False):
             strides, tag, ctypes.byref(cc))
     stream = torch.cuda.current_stream().cuda_stream
     if entry == "static":
+        torch.cuda.synchronize()
+        free0 = torch.cuda.mem_get_info(k.device)[0]
         _lib.call("zp_compress_layers_static", *head, stream)
+        torch.cuda.synchronize()
+        if check_memory:   # nothing was allocated or released on the device, by anyone
+            assert torch.cuda.mem_get_info(k.device)[0] == free0
     else:
         lib = _lib.load()
         need = lib.zp_compress_layers_workspace(L, B, NB, BS, Hkv, Hq, W, tag, ctypes.byref(cc),
@@ -64,15 +70,28 @@ def test_static_scratch_entry_matches_the_workspace_entry(dev, dtype):
     # first call: the larger input; second call: fewer, shorter sequences and other switches
     big, cfg_big = _case(dev, dtype, 5, L=2, B=6, kw=SCRIPTS)
     small, cfg_small = _case(dev, dtype, 6, L=1, B=2, kw=RAW, nb=(3,))
+    from zipage_amd import _lib
+    _lib.call("zp_static_scratch_init")     # the address look-up, outside any capture
     for tensors, cfg in ((big, cfg_big), (small, cfg_small)):
         want = _call("workspace", tensors, cfg)
-        got = _call("static", tensors, cfg)
+        got = _call("static", tensors, cfg, check_memory=True)
         for name, a, b in zip(("flag", "k", "v", "score cache"), got, want):
             assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), name
         assert (got[0].flatten(3).sum(-1) == 2 * 256).all()
         # flags kept inside the library's array: the caches still come out the same
         got2 = _call("static", tensors, cfg, flag_in_scratch=True)
         for name, a, b in zip(("k", "v", "score cache"), got2[1:], want[1:]):
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), name
+
+
+def test_static_scratch_entry_with_the_reference_carry(dev):
+    """deterministic_carry off (the reference's store-then-read-back of the score cache, no page
+    shared in this batch): the same bits as the workspace entry, twice in a row."""
+    tensors, cfg = _case(dev, torch.bfloat16, 8, L=2, B=5, kw=SCRIPTS)
+    for _ in range(2):
+        want = _call("workspace", tensors, cfg, deterministic_carry=False)
+        got = _call("static", tensors, cfg, deterministic_carry=False, check_memory=True)
+        for name, a, b in zip(("flag", "k", "v", "score cache"), got, want):
             assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), name
 
 

@@ -73,6 +73,7 @@ SIGNATURES["zp_compress_layers"] = (
                               C.POINTER(ptr), ptr])
 SIGNATURES["zp_compress_layers_static"] = (
     [ptr] * 9 + [i32] * 11 + [C.POINTER(i64), i32, C.POINTER(CompressConfigC), ptr])
+SIGNATURES["zp_static_scratch_init"] = []
 STATIC_SCRATCH_BYTES = 32 << 20
 I64_RETURNING = {
     "zp_compress_layers_workspace": [i32, i32, i32, i32, i32, i32, i32, i32,

@@ -123,7 +123,9 @@ def compress_layers(k_cache, v_cache, query_cache, score_cache, query_ids, block
     score cache is only read by global_score and the survivors' carried scores are compacted
     straight from the scores it returned: the same values as the reference whenever no page is
     shared, independent of scheduling when one is, and no shared (read-only) page is written.
-    ``False`` runs the reference's two stores.
+    ``False`` runs the reference's two stores.  (The CPU oracle's ``compress_pipeline`` is the
+    reference restated, so ITS default is ``deterministic_carry=False``: a comparison of the two
+    on a batch with shared pages passes the switch explicitly to both.)
     """
     t = timer or StageTimer(False)
     BS = k_cache.shape[2]

@@ -54,11 +54,65 @@ Plan make_plan(int L, int B, int NB, int BS, int Hkv, int Hq, int W, int dtype,
   return p;
 }
 
-int check_config(const zp_compress_config* c) {
+// Everything a stage would refuse is refused here, before the first launch: a chunk either runs
+// all of its stages or none (the global-score stage rewrites the score cache when
+// deterministic_carry is off, so a failure behind it would leave a half-applied step).
+int check_chunk(const zp_compress_config* c, int L, int B, int NB, int BS, int Hkv, int Hq, int D,
+                int W, int target_width, int dtype, bool one_launch_select, const void* score_cache) {
   ZP_REQUIRE(c, "compress_layers: null config");
+  ZP_REQUIRE(L >= 0 && B >= 0 && NB > 0 && BS > 0 && Hkv > 0 && Hq > 0 && D > 0 && W > 0 &&
+                 W <= BS && target_width > 0, "compress_layers: bad dims");
+  ZP_REQUIRE(dtype >= ZP_BF16 && dtype <= ZP_F32, "compress_layers: unknown dtype tag %d", dtype);
+  ZP_REQUIRE(Hq % Hkv == 0, "compress_layers: Hq=%d is not a multiple of Hkv=%d", Hq, Hkv);
   ZP_REQUIRE(c->budget_blocks > 0, "compress_layers: budget_blocks=%d", c->budget_blocks);
-  ZP_REQUIRE(c->query_cache_len > 0, "compress_layers: query_cache_len=%d", c->query_cache_len);
-  ZP_REQUIRE(c->pooling_size >= 0 && c->sink_len >= 0, "compress_layers: negative pooling_size or sink_len");
+  ZP_REQUIRE(c->query_cache_len > 0 && c->query_cache_len <= BS,
+             "compress_layers: query_cache_len=%d outside (0, BS=%d]", c->query_cache_len, BS);
+  ZP_REQUIRE(c->budget_blocks <= NB, "compress_layers: keeping %d pages of a table of %d",
+             c->budget_blocks, NB);
+  ZP_REQUIRE(target_width >= c->budget_blocks, "compress_layers: target table of %d pages for a "
+             "budget of %d", target_width, c->budget_blocks);
+  ZP_REQUIRE(c->reduced == ZP_REDUCE_MEAN || c->reduced == ZP_REDUCE_MAX,
+             "compress_layers: unknown reduction %d", c->reduced);
+  ZP_REQUIRE(c->pooling_size >= 0 && (c->pooling_size <= 1 || (c->pooling_size & 1)),
+             "compress_layers: pooling_size %d must be odd (or 0 / 1 for none)", c->pooling_size);
+  ZP_REQUIRE(c->pooling_mode == ZP_POOL_MAX || c->pooling_mode == ZP_POOL_AVG,
+             "compress_layers: unknown pooling mode %d", c->pooling_mode);
+  ZP_REQUIRE(c->sink_len >= 0, "compress_layers: negative sink_len");
+  if (c->use_global_score) {
+    ZP_REQUIRE(score_cache, "compress_layers: use_global_score needs a score cache");
+    ZP_REQUIRE(c->decay_factor >= 0.f && c->decay_factor <= 1.f,
+               "compress_layers: decay_factor %g outside [0,1]", (double)c->decay_factor);
+    ZP_REQUIRE(c->activate_method == ZP_ACTIVATE_MAX || c->activate_method == ZP_ACTIVATE_SUM,
+               "compress_layers: unknown activate_method %d", c->activate_method);
+  }
+  const int es = zp_dtype_bytes(dtype);
+  const int64_t Tn = (int64_t)NB * BS;
+  if (D > 128 || (D * es) % 16 != 0) {
+    zp_set_error("compress_layers: head_dim %d unsupported (need <= 128 and a multiple of %d)", D, 16 / es);
+    return ZP_EUNSUPPORTED;
+  }
+  const int tile = es == 4 ? 64 : 128;
+  if (BS % tile != 0) {
+    zp_set_error("compress_layers: page size %d is not a multiple of %d", BS, tile);
+    return ZP_EUNSUPPORTED;
+  }
+  int gp = 1;
+  while (gp < Hq / Hkv) gp <<= 1;
+  if (gp > 32) {
+    zp_set_error("compress_layers: GQA group %d unsupported (max 32)", Hq / Hkv);
+    return ZP_EUNSUPPORTED;
+  }
+  ZP_REQUIRE(Tn <= 65536, "compress_layers: NB*BS=%lld exceeds 65536", (long long)Tn);
+  ZP_REQUIRE((int64_t)L * B * Hkv < ((int64_t)1 << 28), "compress_layers: too many (layer, sequence, head) rows");
+  if (!one_launch_select && Tn * 4 > 150 * 1024) {
+    zp_set_error("compress_layers: a row of %lld tokens exceeds what top-k holds in LDS", (long long)Tn);
+    return ZP_EUNSUPPORTED;
+  }
+  if (c->use_redundancy && Tn * (c->lightning ? 4 : 12) > 150 * 1024) {
+    zp_set_error("compress_layers: a row of %lld tokens exceeds what the redundancy softmax holds in LDS",
+                 (long long)Tn);
+    return ZP_EUNSUPPORTED;
+  }
   return ZP_OK;
 }
 
@@ -194,13 +248,6 @@ int run_layers(void* k_cache, void* v_cache, const void* query_cache, void* scor
   return ZP_OK;
 }
 
-int check_dims(int L, int B, int NB, int BS, int Hkv, int Hq, int D, int W, int dtype) {
-  ZP_REQUIRE(L >= 0 && B >= 0 && NB > 0 && BS > 0 && Hkv > 0 && Hq > 0 && D > 0 && W > 0,
-             "compress_layers: bad dims");
-  ZP_REQUIRE(dtype >= ZP_BF16 && dtype <= ZP_F32, "compress_layers: unknown dtype tag %d", dtype);
-  return ZP_OK;
-}
-
 // ---- the library's own scratch: one array per GPU, in that GPU's memory, for the life of the
 // process.  Host code only ever uses the address hipGetSymbolAddress returns for it.
 static __device__ __align__(256) unsigned char scratch[ZP_STATIC_SCRATCH_BYTES];
@@ -233,11 +280,18 @@ int static_scratch(char** out) {
 
 }  // namespace
 
+extern "C" int zp_static_scratch_init(void) {
+  char* ws = nullptr;
+  return static_scratch(&ws);
+}
+
 extern "C" int64_t zp_compress_layers_workspace(int32_t L, int32_t B, int32_t NB, int32_t BS,
                                                 int32_t Hkv, int32_t Hq, int32_t W, int32_t dtype,
                                                 const zp_compress_config* cfg,
                                                 int32_t flag_in_workspace) {
-  if (!cfg || L < 0 || B < 0 || NB <= 0 || BS <= 0 || Hkv <= 0 || Hq <= 0 || W <= 0) return -1;
+  if (!cfg || L < 0 || B < 0 || NB <= 0 || BS <= 0 || Hkv <= 0 || Hq <= 0 || W <= 0 ||
+      dtype < ZP_BF16 || dtype > ZP_F32)
+    return -1;
   return make_plan(L, B, NB, BS, Hkv, Hq, W, dtype, cfg, flag_in_workspace != 0).total;
 }
 
@@ -251,9 +305,9 @@ extern "C" int zp_compress_layers(void* k_cache, void* v_cache, const void* quer
                                   int32_t dtype, const zp_compress_config* cfg, void* workspace,
                                   int64_t workspace_bytes, void* const* stage_events,
                                   void* stream) {
-  int rc = check_dims(L, B, NB, BS, Hkv, Hq, D, W, dtype);
-  if (rc != ZP_OK) return rc;
-  rc = check_config(cfg);
+  ZP_REQUIRE(cfg, "compress_layers: null config");
+  int rc = check_chunk(cfg, L, B, NB, BS, Hkv, Hq, D, W, target_width, dtype,
+                       select_fits((int64_t)NB * BS), score_cache);
   if (rc != ZP_OK) return rc;
   ZP_REQUIRE(k_cache && v_cache && query_cache && seq_idx && block_table && compressed &&
                  target_block_table && strides, "compress_layers: null pointer");
@@ -278,9 +332,9 @@ extern "C" int zp_compress_layers_static(void* k_cache, void* v_cache, const voi
                                          int32_t target_width, const int64_t* strides,
                                          int32_t dtype, const zp_compress_config* cfg,
                                          void* stream) {
-  int rc = check_dims(L, B, NB, BS, Hkv, Hq, D, W, dtype);
-  if (rc != ZP_OK) return rc;
-  rc = check_config(cfg);
+  ZP_REQUIRE(cfg, "compress_layers_static: null config");
+  int rc = check_chunk(cfg, L, B, NB, BS, Hkv, Hq, D, W, target_width, dtype,
+                       select_fits((int64_t)NB * BS), score_cache);
   if (rc != ZP_OK) return rc;
   ZP_REQUIRE(k_cache && v_cache && query_cache && seq_idx && block_table && compressed &&
                  target_block_table && strides, "compress_layers_static: null pointer");
