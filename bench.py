@@ -78,7 +78,7 @@ def cpu_baseline(wl, cfg, sample_seqs, layers=1, budget_s=30.0):
 
 
 def end_to_end(requests=256, prompt=512, out_tokens=4096, async_compress=True, ragged=False,
-               script_switches=False):
+               script_switches=False, attention_probe=True):
     """BASELINE configs[4]: offline decode of a random-init Qwen3-8B with the KV budget on.
     Returns decode tokens/s (decode steps only, first decode step to the last, device-complete),
     the share of that time the compression kernels were running, and the bandwidth of the
@@ -105,6 +105,26 @@ def end_to_end(requests=256, prompt=512, out_tokens=4096, async_compress=True, r
     outs = eng.generate(prompts, SamplingParams(max_tokens=out_tokens, ignore_eos=True))
     st = eng.stats
     assert all(len(o["token_ids"]) == out_tokens for o in outs)
+    out = {
+        "workload": (f"configs[4]: random-init Qwen3-8B bf16, {requests} requests, "
+                     f"{'ragged ' if ragged else ''}{prompt}-token prompts"
+                     + (f" (uniform in [{prompt // 2}, {prompt + prompt // 2}])" if ragged else "")
+                     + f", {out_tokens} greedy tokens "
+                     "each, budget 8 pages x 256 tokens, window 16, "
+                     + ("global score (decay 0.8) + lightning redundancy + max-pool 5" if script_switches
+                        else "max-pool 5") + ", compression "
+                     + ("on a side stream" if async_compress else "in line with the decode steps")),
+        "decode_tok_per_s": round(st["decode_tokens"] / st["decode_s"], 1),
+        "ms_per_decode_step": round(st["decode_s"] / st["decode_steps"] * 1e3, 3),
+        "decode_steps": st["decode_steps"],
+        "prefill_tok_per_s": round(st["prefill_tokens"] / st["prefill_s"], 1),
+        "compress_calls": st["compress_calls"], "sequences_compressed": st["compress_seqs"],
+        "compress_share_of_decode_time": round(st["compress_s"] / st["decode_s"], 5),
+    }
+    if not attention_probe:
+        del eng
+        torch.cuda.empty_cache()
+        return out
     # decode attention alone, at the steady-state shape of this run (8 full pages + half a page)
     r = eng.runner
     B, BS = requests, cfg.kvcache_block_size
@@ -123,24 +143,12 @@ def end_to_end(requests=256, prompt=512, out_tokens=4096, async_compress=True, r
     torch.cuda.synchronize()
     us = e0.elapsed_time(e1) / 20 * 1e3
     alg = B * ctx_len * QWEN3_8B.kv_heads * QWEN3_8B.head_dim * 2 * 2   # K and V rows, read once
-    out = {
-        "workload": (f"configs[4]: random-init Qwen3-8B bf16, {requests} requests, "
-                     f"{'ragged ' if ragged else ''}{prompt}-token prompts, {out_tokens} greedy tokens "
-                     "each, budget 8 pages x 256 tokens, window 16, "
-                     + ("global score (decay 0.8) + lightning redundancy + max-pool 5" if script_switches
-                        else "max-pool 5") + ", compression "
-                     + ("on a side stream" if async_compress else "in line with the decode steps")),
-        "decode_tok_per_s": round(st["decode_tokens"] / st["decode_s"], 1),
-        "ms_per_decode_step": round(st["decode_s"] / st["decode_steps"] * 1e3, 3),
-        "decode_steps": st["decode_steps"],
-        "prefill_tok_per_s": round(st["prefill_tokens"] / st["prefill_s"], 1),
-        "compress_calls": st["compress_calls"], "sequences_compressed": st["compress_seqs"],
-        "compress_share_of_decode_time": round(st["compress_s"] / st["decode_s"], 5),
+    out.update({
         "decode_attention": {"bound": "hbm", "kernel": "paged_decode_kernel",
                              "avg_launch_us": round(us, 1), "algorithmic_bytes": alg,
                              "achieved": round(alg / us / 1e3, 1), "peak": HBM_PEAK_GBS,
                              "unit": "GB/s", "frac": round(alg / us / 1e3 / HBM_PEAK_GBS, 4)},
-    }
+    })
     del eng
     torch.cuda.empty_cache()
     return out
@@ -338,6 +346,11 @@ def main():
                     help="skip the end-to-end decode leg that follows the default run")
     ap.add_argument("--no-extra-legs", action="store_true",
                     help="skip the 64-sequence leg and the end-to-end leg that follow the default run")
+    ap.add_argument("--no-e2e-variants", action="store_true",
+                    help="skip the four shorter end-to-end runs (reference scripts' switches / ragged "
+                         "prompts, each with side-stream and in-line compression)")
+    ap.add_argument("--variant-tokens", type=int, default=2560,
+                    help="greedy tokens per request in the end-to-end variants")
     ap.add_argument("--requests", type=int, default=256)
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--out-tokens", type=int, default=4096)
@@ -425,6 +438,14 @@ def main():
             out["end_to_end"] = end_to_end(args.requests, args.prompt, args.out_tokens,
                                            not args.sync_compress, args.ragged_prompts,
                                            args.script_switches)
+            if not args.no_e2e_variants:
+                # where overlap can exist and where the compression does more work: the reference
+                # scripts' switch set and ragged prompts, each on the side stream and in line,
+                # from this same process (shorter runs: every sequence still compresses 2-4 times)
+                n = min(args.out_tokens, args.variant_tokens)
+                out["end_to_end"]["variants"] = [
+                    end_to_end(args.requests, args.prompt, n, a, ragged, scripts, attention_probe=False)
+                    for scripts, ragged in ((True, False), (False, True)) for a in (True, False)]
     print(json.dumps(out))
 
 

@@ -340,6 +340,226 @@ __global__ __launch_bounds__(NW * 64) void gram_kernel(GramArgs p) {
   }
 }
 
+// ------------------------------------------------------------------ fp32 caches, raw, every pair of pages once
+// One workgroup per (layer, sequence, head, valid page a), pages of at most 256 keys.  The
+// similarity matrix of a sequence is symmetric, so page a multiplies its rows only with the pages
+// (a + d) mod n, d = 0 .. n/2 (the pairs at distance n/2 go to the lower half of the pages when n
+// is even).  A tile off the diagonal page serves both of its sides: the rows get their partial
+// row sums and their claim (last column over the threshold) as in gram_kernel; the columns get
+// the tile's column sums -- slot [d][key], written by exactly one workgroup and added in a fixed
+// order by the softmax kernel -- and the last ROW over the threshold as their claim.  Claims meet
+// in one 64-bit word per key, (index + 1) << 32 | value bits, through atomicMax: the largest
+// index wins whatever the order of the workgroups.
+constexpr int kSymWaves = 8;
+constexpr int kSymMaxDist = 8;      // column-sum slots per key the workspace holds: tables of <= 16 pages
+
+__global__ void fill_u64_kernel(unsigned long long* dst, int64_t n, unsigned long long v) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = v;
+}
+
+__global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramArgs p) {
+  typedef F32 T;
+  constexpr int kThreads = kSymWaves * 64;
+  constexpr int PIECES = kDmax / 4;                 // 16-byte pieces per key row
+  constexpr int ROWS_PER_IT = kThreads / PIECES;    // 16
+  constexpr int STAGE_IT = TN / ROWS_PER_IT;        // 4
+  constexpr int NSUB = TN / 32;
+
+  extern __shared__ __align__(16) char smem[];
+  float* kbuf0 = (float*)smem;
+  float* kbuf1 = kbuf0 + TN * ROWF;
+  float* l_cpart = kbuf1 + TN * ROWF;               // [2][kSymWaves][TN] column sums per wave and tile
+  int* vpage = (int*)(l_cpart + 2 * kSymWaves * TN);
+  int* vidx = vpage + p.NB;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, col = lane & 31;
+  const int jp = blockIdx.x % p.NB;
+  const int h = (blockIdx.x / p.NB) % p.Hkv;
+  const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
+  const int l = blockIdx.x / (p.NB * p.Hkv * p.B);
+  const int Tn = p.NB * p.BS;
+  const int64_t obase = (((int64_t)l * p.B + b) * p.Hkv + h) * Tn;
+  unsigned long long* ws_claim = (unsigned long long*)p.ws_col;   // (rows, Tn) words of 64 bits
+  const int64_t n_keys = (int64_t)gridDim.x * p.BS;               // == L * B * Hkv * Tn
+
+  const int code = p.table[(int64_t)b * p.NB + jp];
+  int rpid = page_is_pad(code) ? -1 : page_id(code);
+  if (rpid >= p.num_pages) rpid = -1;
+  if (rpid < 0) return;
+
+  __shared__ int nvalid_s, mine_s;
+  if (tid == 0) {
+    int n = 0, me = 0;
+    for (int j = 0; j < p.NB; ++j) {
+      const int c = p.table[(int64_t)b * p.NB + j];
+      const int pid = page_is_pad(c) ? -1 : page_id(c);
+      if (pid >= 0 && pid < p.num_pages) {
+        if (j == jp) me = n;
+        vpage[n] = pid; vidx[n] = j; ++n;
+      }
+    }
+    nvalid_s = n; mine_s = me;
+  }
+  for (int i = tid; i < 2 * TN * ROWF; i += kThreads) kbuf0[i] = 0.f;
+  __syncthreads();
+  const int n = nvalid_s, ai = mine_s;
+  const int nd = n / 2 + (((n & 1) || ai < n / 2) ? 1 : 0);     // distances 0 .. nd-1
+  const int tiles_per_page = p.BS / TN;
+  const int ntiles = nd * tiles_per_page;
+  const int dpieces = p.D / 4;
+  const int64_t k_row = (int64_t)p.Hkv * p.D * 4;
+  const char* kbase = p.k + (l * p.k_sl) * 4 + (int64_t)h * p.D * 4;
+
+  const int st_piece = tid % PIECES, st_row0 = tid / PIECES;
+  vec16 pre[STAGE_IT];
+  auto col_page = [&](int d) { return ai + d < n ? ai + d : ai + d - n; };
+  auto issue_loads = [&](int tile) {
+    const int d = tile / tiles_per_page, toff = (tile - d * tiles_per_page) * TN;
+    const char* src = kbase + (int64_t)vpage[col_page(d)] * p.k_sp * 4 + (int64_t)toff * k_row;
+#pragma unroll
+    for (int i = 0; i < STAGE_IT; ++i) {
+      const int row = st_row0 + i * ROWS_PER_IT;
+      pre[i] = vec16{0u, 0u, 0u, 0u};
+      if (st_piece < dpieces) pre[i] = *(const vec16*)(src + (int64_t)row * k_row + st_piece * 16);
+    }
+  };
+  auto commit_loads = [&](float* buf) {
+#pragma unroll
+    for (int i = 0; i < STAGE_IT; ++i) {
+      const int row = st_row0 + i * ROWS_PER_IT;
+      float e[4];
+      Unpack<T>::run(pre[i], e);
+      float ss = (e[0] * e[0] + e[1] * e[1]) + (e[2] * e[2] + e[3] * e[3]);
+      ss = pieces_sum<PIECES>(ss);
+      const float rn = __builtin_amdgcn_rcpf(fmaxf(__builtin_amdgcn_sqrtf(ss), p.eps));
+      if (st_piece < dpieces)
+        *(float4*)(buf + row * ROWF + st_piece * 4) = make_float4(e[0] * rn, e[1] * rn, e[2] * rn, e[3] * rn);
+    }
+  };
+
+  const int row_blocks = p.BS / 32;
+  const int rb = wave;
+  const bool active = rb < row_blocks;
+  // A fragments: this lane's key row of page a, normalised; k-step 4j + i of wave half `half` takes
+  // element 8j + 4 half + i (the same order as the B operand's 16-byte LDS reads)
+  float afrag[KS];
+  {
+    const int slot = (active ? rb : 0) * 32 + col;
+    const char* src = kbase + (int64_t)rpid * p.k_sp * 4 + (int64_t)slot * k_row;
+    float ss = 0.f;
+#pragma unroll
+    for (int pc = 0; pc < PIECES; ++pc) {
+      float e[4];
+      vec16 v = vec16{0u, 0u, 0u, 0u};
+      if (pc < dpieces) v = *(const vec16*)(src + pc * 16);
+      Unpack<T>::run(v, e);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) ss += e[q] * e[q];
+      if ((pc & 1) == 0) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) afrag[(pc >> 1) * 4 + q] = e[q];
+      } else if (half) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) afrag[(pc >> 1) * 4 + q] = e[q];
+      }
+    }
+    const float rn = __builtin_amdgcn_rcpf(fmaxf(__builtin_amdgcn_sqrtf(ss), p.eps));
+#pragma unroll
+    for (int s = 0; s < KS; ++s) afrag[s] = active ? afrag[s] * rn : 0.f;
+  }
+  float rsum[16], cval[16];
+  int ccol[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) { rsum[r] = 0.f; cval[r] = 0.f; ccol[r] = -1; }
+
+  // the column sums of tile t are complete after the barrier that ends it: the waves' shares are
+  // added in wave order and stored while tile t+1 is being multiplied
+  auto finish_columns = [&](int tile) {
+    const int d = tile / tiles_per_page, toff = (tile - d * tiles_per_page) * TN;
+    if (d == 0 || tid >= TN) return;
+    const float* pt = l_cpart + (tile & 1) * kSymWaves * TN;
+    float v = pt[tid];
+#pragma unroll
+    for (int w2 = 1; w2 < kSymWaves; ++w2) v += pt[w2 * TN + tid];
+    const int jc = vidx[col_page(d)];
+    p.ws_chunk[(int64_t)(d - 1) * n_keys + obase + (int64_t)jc * p.BS + toff + tid] = v;
+  };
+
+  if (ntiles > 0) { issue_loads(0); commit_loads(kbuf0); }
+  __syncthreads();
+  for (int tile = 0; tile < ntiles; ++tile) {
+    float* cur = (tile & 1) ? kbuf1 : kbuf0;
+    float* nxt = (tile & 1) ? kbuf0 : kbuf1;
+    if (tile + 1 < ntiles) issue_loads(tile + 1);
+    const int d = tile / tiles_per_page, toff = (tile - d * tiles_per_page) * TN;
+    const int jc = vidx[col_page(d)];
+    float* cpart = l_cpart + ((tile & 1) * kSymWaves + wave) * TN;
+#pragma unroll
+    for (int st = 0; st < NSUB; ++st) {
+      float csum = 0.f, rv = 0.f;
+      int rlast = -1;
+      if (active) {
+        f32x16_t acc;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        const float4* b4 = (const float4*)(cur + (st * 32 + col) * ROWF + 4 * half);
+#pragma unroll
+        for (int j4 = 0; j4 < KS / 4; ++j4) {
+          const float4 bv = b4[2 * j4];
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 0], bv.x, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 1], bv.y, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 2], bv.z, acc, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 3], bv.w, acc, 0, 0, 0);
+        }
+        const int cslot = toff + st * 32 + col;
+        const int cidx = jc * p.BS + cslot;   // logical index of this lane's column key
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+          float sv = acc[r];
+          if (d == 0 && rslot == cslot) sv = 0.f;
+          rsum[r] += sv;
+          csum += sv;
+          const bool over = sv > p.threshold;
+          if (over && cidx > ccol[r]) { ccol[r] = cidx; cval[r] = sv; }
+          if (over) { rlast = rslot; rv = sv; }   // rslot grows with r inside a lane
+        }
+        if (d != 0) {
+          const int orl = lane_xor32(rlast);
+          const float orv = lane_xor32(rv);
+          if (orl > rlast) { rlast = orl; rv = orv; }
+          if (half == 0 && rlast >= 0)   // rare: the column key's claim candidate among page a's rows
+            atomicMax(&ws_claim[obase + cidx],
+                      ((unsigned long long)(unsigned)(jp * p.BS + rlast + 1) << 32) | __float_as_uint(rv));
+        }
+      }
+      if (d != 0) {
+        csum += lane_xor32(csum);
+        if (half == 0) cpart[st * 32 + col] = csum;
+      }
+    }
+    if (tile + 1 < ntiles) commit_loads(nxt);
+    __syncthreads();
+    finish_columns(tile);
+  }
+  // ---- row side: sums and claims over the 32 lanes of each half
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float sv = half_sum(rsum[r]);
+    int c = ccol[r];
+    float v = cval[r];
+    last_claim_reduce(c, v);
+    if (active && col == 0) {
+      const int64_t oi = obase + (int64_t)jp * p.BS + rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+      p.ws_sum[oi] = sv;
+      if (c >= 0)
+        atomicMax(&ws_claim[oi], ((unsigned long long)(unsigned)(c + 1) << 32) | __float_as_uint(v));
+    }
+  }
+}
+
 // ------------------------------------------------------------------ fp32 caches, lightning, whole page in LDS
 // One workgroup per (layer, sequence, head, page) of at most 256 keys: the page is loaded once
 // with coalesced 16-byte loads, normalised on the way into LDS (132 KB), and after ONE barrier
@@ -1591,7 +1811,10 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
     const float* __restrict__ ws_sum, const int32_t* __restrict__ ws_col,
     const float* __restrict__ ws_val, int B, int NB, int BS, int Hkv, int num_pages,
     float tscale /* raw: temperature; lightning: temperature*BS */,
-    int rows_ready /* raw: the row sums are already in `red` (16-bit caches) */) {
+    int rows_ready /* raw: the row sums are already in `red` (16-bit caches) */,
+    const float* __restrict__ ws_csum = nullptr /* raw, fp32, every pair of pages once: column-side
+        sums [distance - 1][row][Tn]; ws_col then holds 64-bit (index + 1, value) claims */,
+    int64_t n_keys = 0) {
   extern __shared__ __align__(16) char smem[];
   __shared__ float red_lds[kWaves];
   const int Tn = NB * BS;
@@ -1610,6 +1833,7 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
     nvalid += (pid >= 0 && pid < num_pages) ? 1 : 0;
   }
   const float divisor = RAW ? tscale * (float)(nvalid * BS) : tscale;
+  const unsigned long long* claims = (const unsigned long long*)ws_col;
   if (from_ws) {
     // every key hands the value of its claimed entry to the row it was taken from: 2^-32 fixed
     // point with integer atomics, exact and independent of the order
@@ -1619,8 +1843,14 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
       const int c = trow[t / BS];
       const int pid = page_is_pad(c) ? -1 : page_id(c);
       if (pid < 0 || pid >= num_pages) continue;
-      const int cc = ws_col[base + t];
-      if (cc >= 0 && cc < Tn) atomicAdd(&corr[cc], to_fixed32(ws_val[base + t]));
+      if (ws_csum) {
+        const unsigned long long cl = claims[base + t];
+        const int cc = (int)(cl >> 32) - 1;
+        if (cc >= 0 && cc < Tn) atomicAdd(&corr[cc], to_fixed32(__uint_as_float((unsigned)cl)));
+      } else {
+        const int cc = ws_col[base + t];
+        if (cc >= 0 && cc < Tn) atomicAdd(&corr[cc], to_fixed32(ws_val[base + t]));
+      }
     }
     __syncthreads();
   }
@@ -1631,7 +1861,23 @@ __global__ __launch_bounds__(kThreads) void red_softmax_kernel(
       const int c = trow[t / BS];
       const int pid = page_is_pad(c) ? -1 : page_id(c);
       if (pid >= 0 && pid < num_pages) {
-        r = Elem<T>::rnd(ws_sum[base + t] - from_fixed32(corr[t]));
+        float sv = ws_sum[base + t];
+        if (ws_csum) {
+          // the column-side sums of this key's page: distance d was written by the valid page
+          // d places before it (cyclically), if that page ran the distance
+          int ci = 0;
+          for (int j = 0; j < t / BS; ++j) {
+            const int c2 = trow[j];
+            const int p2 = page_is_pad(c2) ? -1 : page_id(c2);
+            ci += (p2 >= 0 && p2 < num_pages) ? 1 : 0;
+          }
+          for (int d = 1; d <= nvalid / 2; ++d) {
+            const int a = ci - d >= 0 ? ci - d : ci - d + nvalid;
+            const bool ran = d < nvalid / 2 + (((nvalid & 1) || a < nvalid / 2) ? 1 : 0);
+            if (ran) sv += ws_csum[(int64_t)(d - 1) * n_keys + base + t];
+          }
+        }
+        r = Elem<T>::rnd(sv - from_fixed32(corr[t]));
       } else {
         r = -INFINITY;
       }
@@ -1759,7 +2005,8 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
 template <typename T, bool RAW>
 int launch_softmax(void* red, void* logits, const int32_t* table, const float* ws_sum,
                    const int32_t* ws_col, const float* ws_val, int L, int B, int NB, int BS,
-                   int Hkv, int num_pages, double temperature, hipStream_t st, int rows_ready = 0) {
+                   int Hkv, int num_pages, double temperature, hipStream_t st, int rows_ready = 0,
+                   const float* ws_csum = nullptr) {
   const size_t smem = (size_t)NB * BS * ((RAW && !rows_ready) ? 12 : 4);
   if (smem > 150 * 1024) {
     zp_set_error("redundancy: a row of %d tokens exceeds LDS", NB * BS);
