@@ -1921,6 +1921,12 @@ int check_common(const char* name, const void* k_cache, const int32_t* table, vo
   return ZP_OK;
 }
 
+// fp32 all-pairs: can every unordered pair of pages be multiplied once (pages of at most 256
+// keys in whole 64-key tiles, column-sum slots for every distance in the workspace)?
+inline bool raw_f32_symmetric(int NB, int BS) {
+  return BS <= 256 && BS % TN == 0 && NB / 2 <= kSymMaxDist;
+}
+
 template <typename T, bool RAW>
 int launch_gram(const GramArgs& a, int L, hipStream_t st) {
   dim3 grid((unsigned)((int64_t)L * a.B * a.Hkv * a.NB));
@@ -1948,6 +1954,22 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
         return ZP_EHIP;
       }
       hipLaunchKernelGGL(gram_page_f32_kernel, grid, dim3(kPage32Threads), smem, st, a);
+      ZP_LAUNCH_CHECK();
+      return ZP_OK;
+    }
+  }
+  if constexpr (T::bytes == 4 && RAW) {
+    if (raw_f32_symmetric(a.NB, a.BS)) {
+      const int64_t n = (int64_t)L * a.B * a.Hkv * a.NB * a.BS;
+      const size_t smem = sizeof(float) * (2 * TN * ROWF + 2 * kSymWaves * TN) + sizeof(int) * 2 * a.NB;
+      if (hipFuncSetAttribute((const void*)gram_raw_sym_f32_kernel,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
+        zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
+        return ZP_EHIP;
+      }
+      hipLaunchKernelGGL(fill_u64_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                         (unsigned long long*)a.ws_col, n, 0ull);
+      hipLaunchKernelGGL(gram_raw_sym_f32_kernel, grid, dim3(kSymWaves * 64), smem, st, a);
       ZP_LAUNCH_CHECK();
       return ZP_OK;
     }
@@ -2021,7 +2043,8 @@ int launch_softmax(void* red, void* logits, const int32_t* table, const float* w
   dim3 grid((unsigned)((int64_t)L * B * Hkv));
   hipLaunchKernelGGL((red_softmax_kernel<T, RAW>), grid, dim3(kThreads), smem, st, red, logits,
                      table, ws_sum, ws_col, ws_val, B, NB, BS, Hkv, num_pages,
-                     RAW ? (float)temperature : (float)(temperature * (double)BS), rows_ready);
+                     RAW ? (float)temperature : (float)(temperature * (double)BS), rows_ready,
+                     ws_csum, (int64_t)L * B * Hkv * NB * BS);
   ZP_LAUNCH_CHECK();
   return ZP_OK;
 }
@@ -2085,7 +2108,8 @@ extern "C" int zp_redundancy_raw(const void* k_cache, const int32_t* block_table
     rc = launch_gram<T, true>(a, L, st);
     if (rc != ZP_OK) return rc;
     rc = launch_softmax<T, true>(red_out, logits_out, block_table, a.ws_sum, a.ws_col, a.ws_val, L,
-                                 B, NB, BS, Hkv, num_pages, temperature, st, T::bytes == 2);
+                                 B, NB, BS, Hkv, num_pages, temperature, st, T::bytes == 2,
+                                 (T::bytes == 4 && raw_f32_symmetric(NB, BS)) ? a.ws_chunk : nullptr);
   });
   return rc;
 }
