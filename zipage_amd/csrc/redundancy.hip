@@ -1654,7 +1654,10 @@ __global__ __launch_bounds__(512) void raw_chain_kernel(GramArgs p) {
   int* cl = (int*)(smem + 3 * CT * ROWH);                // [CT][KEYS] corrections, then chunk sums
   int* vidx = cl + CT * KEYS;                            // [NB] logical page of the n-th valid page
   int* vord = vidx + p.NB;                               // [NB] inverse (-1: pad)
-  __shared__ int nvalid_s;
+  // the claims taken from this round's keys, gathered once per round: (chunk << 16 | key) and value
+  uint32_t* lst_key = (uint32_t*)(vord + p.NB);          // [NB * BS]
+  float* lst_val = (float*)(lst_key + (size_t)p.NB * p.BS);
+  __shared__ int nvalid_s, nlist_s;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
@@ -1718,6 +1721,25 @@ __global__ __launch_bounds__(512) void raw_chain_kernel(GramArgs p) {
     const float diag = ssq * rn * rn;                 // S_ii, the entry the reference zeroes
     const int own_chunk = my_ord * cpp + slot / kChunk;
     float part = 0.f, total = 0.f;                    // chain state of key `tid` (tid < KEYS)
+    // every key of the sequence claims at most one entry: one pass over the claims keeps those
+    // taken from this round's keys, with the chunk of the claiming key (the order of the list does
+    // not matter, the values are added as fixed point)
+    __syncthreads();
+    if (tid == 0) nlist_s = 0;
+    __syncthreads();
+    for (int t = tid; t < Tn; t += kT) {
+      const int jt = t / p.BS;
+      const int ord = vord[jt];
+      if (ord < 0) continue;
+      const int cc = p.ws_col[obase + t] - (jp * p.BS + key0);   // the row key t claimed from
+      if (cc >= 0 && cc < KEYS && key0 + cc < p.BS) {
+        const int i = atomicAdd(&nlist_s, 1);
+        lst_key[i] = (uint32_t)(ord * cpp + (t - jt * p.BS) / kChunk) << 16 | (uint32_t)cc;
+        lst_val[i] = p.ws_val[obase + t];
+      }
+    }
+    __syncthreads();
+    const int nlist = nlist_s;
 
     for (int tile = 0; tile < ntiles; ++tile) {
       const int c0 = tile * CT;
@@ -1746,15 +1768,11 @@ __global__ __launch_bounds__(512) void raw_chain_kernel(GramArgs p) {
       __syncthreads();
       if (half == 0 && live && own_chunk >= c0 && own_chunk < c0 + CT)
         atomicAdd(&cl[(own_chunk - c0) * KEYS + wave * 32 + col], to_fixed26(diag));
-      for (int t = tid; t < Tn; t += kT) {
-        const int jt = t / p.BS;
-        const int ord = vord[jt];
-        if (ord < 0) continue;
-        const int vc = ord * cpp + (t - jt * p.BS) / kChunk;
-        if (vc < c0 || vc >= c0 + CT) continue;
-        const int cc = p.ws_col[obase + t] - (jp * p.BS + key0);   // the row key t claimed from
-        if (cc >= 0 && cc < KEYS && key0 + cc < p.BS)
-          atomicAdd(&cl[(vc - c0) * KEYS + cc], to_fixed26(p.ws_val[obase + t]));
+      for (int i = tid; i < nlist; i += kT) {
+        const uint32_t w = lst_key[i];
+        const int vc = (int)(w >> 16);
+        if (vc >= c0 && vc < c0 + CT)
+          atomicAdd(&cl[(vc - c0) * KEYS + (int)(w & 0xffffu)], to_fixed26(lst_val[i]));
       }
       __syncthreads();
       // ---- chunk sums of the tile: A = planes (rows = chunks), B = keys
@@ -1980,7 +1998,12 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
     const size_t smem1 = 2 * (size_t)tn * ROWH + sizeof(int) * 4 * tn + sizeof(float) * a.BS +
                          sizeof(int) * 2 * a.NB;
     const void* fn = tn == 128 ? (const void*)gram_raw_kernel<T, 128> : (const void*)gram_raw_kernel<T, TN>;
-    const size_t smem2 = 3 * 32 * (size_t)ROWH + sizeof(int) * 32 * 256 + sizeof(int) * 2 * a.NB;
+    const size_t smem2 = 3 * 32 * (size_t)ROWH + sizeof(int) * 32 * 256 + sizeof(int) * 2 * a.NB +
+                         (size_t)a.NB * a.BS * 8;   // + the round's claim list
+    if (smem2 > 160 * 1024) {
+      zp_set_error("redundancy: a row of %d tokens exceeds LDS", a.NB * a.BS);
+      return ZP_EUNSUPPORTED;
+    }
     if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1) != hipSuccess ||
         hipFuncSetAttribute((const void*)raw_chain_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)smem2) != hipSuccess) {
