@@ -1,27 +1,33 @@
 // Ragged attention scorer: softmax(window queries x paged keys), max over the GQA group,
-// mean (or max) over the window -- one workgroup per (layer, sequence, kv head), MFMA
-// for the QK^T contraction, K tiles staged through double-buffered LDS.
-//
-// The (Hq, W, T) logits the reference materialises are never written (unless the caller
-// asks for them).  The softmax normaliser spans the whole sequence, so the workgroup makes
-// three passes over the sequence's pages, recomputing QK^T each time:
-//   pass 1  row maximum of the (rounded) logits,
-//   pass 2  row sum of exp(rounded(logit - max)),
-//   pass 3  p = exp(.) / sum, max over the group, sum over the window, store (the group
-//           maximum is taken on the exponents x*log2(e) - log2(sum), one exponential per group).
-// Passes 2 and 3 re-read K from L2 / Infinity Cache.  Rounding points follow the
-// reference (logits, logit-max, softmax output and the window mean are each rounded to the
-// cache dtype), so bf16/fp16 results agree with it to the last bit except where fp32
+// mean (or max) over the window, MFMA for the QK^T contraction.  The (Hq, W, T) logits the
+// reference materialises are never written (unless the caller asks for them).  Rounding points
+// follow the reference (logits, logit - max, softmax output and the window mean are each rounded
+// to the cache dtype), so bf16/fp16 results agree with it to the last bit except where fp32
 // accumulation order moves a value across a rounding boundary.
 //
-// MFMA tiling (wave64, 32x32 tiles): the A operand is a block of 32 query rows, row
-// m = w*Gp + g (Gp = GQA group padded to a power of two), held in registers for the
-// whole pass; the B operand is 32 tokens of the K tile read from LDS.  In the 32x32
-// accumulator layout a lane owns one token column and 16 rows
-// ((r/4)*8 + (lane/32)*4 + r%4), so with this row order the group maximum is taken inside
-// a lane (plus one cross-half exchange when Gp >= 8) and the window sum is a lane-local
-// sum plus one cross-half and one cross-wave (LDS) step.  Wave v of the workgroup owns
-// row block v; tiles of 128 (16-bit) or 64 (fp32) tokens are shared by all waves.
+// Two kernels:
+//   score_resident_kernel  16-bit caches, at most 2560 tokens per sequence, no logits requested:
+//       ONE sweep over K.  A workgroup is one block of 32 query rows of a (layer, sequence, head);
+//       its rounded logits stay in registers (two per word) and the row maximum, the row sum and
+//       the output come from the registers.  Described above the kernel.
+//   score_kernel           everything else (fp32 caches, longer sequences, logits, no scratch):
+//       one workgroup per (layer, sequence, kv head).  The softmax normaliser spans the whole
+//       sequence, so it makes three passes over the sequence's pages, recomputing QK^T each time:
+//         pass 1  row maximum of the (rounded) logits,
+//         pass 2  row sum of exp(rounded(logit - max)),
+//         pass 3  p = exp(.) / sum, max over the group, sum over the window, store (the group
+//                 maximum is taken on the exponents x*log2(e) - log2(sum), one exponential per
+//                 group).
+//       fp32 caches take passes 1 and 2 in one sweep.  K tiles are staged through double-buffered
+//       LDS; passes 2 and 3 re-read K from L2 / Infinity Cache.
+//
+// MFMA tiling (wave64, 32x32 tiles), both kernels: the A operand is a block of 32 query rows, row
+// m = w*Gp + g (Gp = GQA group padded to a power of two), held in registers; the B operand is 32
+// tokens of K read from LDS.  In the 32x32 accumulator layout a lane owns one token column and
+// 16 rows ((r/4)*8 + (lane/32)*4 + r%4), so with this row order the group maximum is taken inside
+// a lane (plus one cross-half exchange when Gp >= 8) and the window sum is a lane-local sum plus
+// one cross-half step; the row blocks' shares meet in LDS (score_kernel: wave v owns row block v,
+// tiles of 128 or 64 tokens are shared by all waves) or in the scratch (score_resident_kernel).
 #include "common.h"
 #include <math.h>
 #include <type_traits>
