@@ -23,6 +23,7 @@
 //                      accumulated in the cache dtype chunk by chunk as the reference does.
 //   red_softmax_kernel claim corrections of the raw variant and the softmax of both.
 #include "common.h"
+#include <type_traits>
 #include <math.h>
 
 namespace {
@@ -1039,26 +1040,72 @@ template <> struct Split3<F16> {
 
 // The cosine matrix factors as S_ij = rn_i rn_j (k_i . k_j) with rn = 1 / norm: the raw 16-bit
 // keys go to the matrix cores as they are (one MFMA per k-step, exact products, fp32 sums) and
-// the two scale factors are applied to the accumulators.  One plane of raw keys in LDS (68 KB),
-// so two workgroups share a compute unit and one's page load hides behind the other's tiles.
+// the two scale factors are applied to the accumulators.  Sixteen waves share a compute unit's
+// four vector units, and vector instruction issue is the first thing they run out of, so
+// everything that can be is kept off the vector ALUs:
+//   * the page goes from global memory straight into LDS (no staging registers, no LDS stores);
+//     a load instruction moves four key rows, which sit 1040 bytes apart in groups of four so that
+//     the matrix cores' fragment reads spread over the banks: piece g (16 bytes) of row r of a
+//     group at (g / 4) * 256 + r * 64 + (g % 4) * 16;
+//   * wave a loads row block a, so it can take the block's norms from the diagonal of its own
+//     Gram tile (which the claim rule needs anyway) before any barrier;
+//   * the summed normalised key  sum_j rn_j k_j  is a matrix product too, contracted over the
+//     keys: A = rn as three 16-bit pieces (rows 0..2), B = the keys read through the transposing
+//     LDS load (`ds_read_b64_tr_b16`: lane i of sixteen receives column i of a 4 x 16 block).
+// One plane of raw keys in LDS (65 KB), so two workgroups share a compute unit.
+constexpr int kPgGrp = 1040;                          // bytes from one group of four key rows to the next
+constexpr int kPgBytes = (kPageRows / 4) * kPgGrp;    // the page in LDS
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x8_t __attribute__((ext_vector_type(8)));
+typedef void __attribute__((address_space(3))) * lds_ptr_t;
+
+#ifdef ZP_PAGE_STAMP
+// Measurement build: thread 0 of every workgroup records the core-clock counter at the phase
+// boundaries and the constant-rate counter at both ends.
+constexpr int kPageStampMax = 1 << 16;
+__device__ long long zp_page_stamp_buf[kPageStampMax * 12];
+extern "C" int zp_debug_page_stamps(long long* dst, int n_groups) {
+  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(zp_page_stamp_buf), (size_t)n_groups * 12 * 8);
+}
+#define ZP_PSTAMP() do { if (tid == 0 && nst < 10) st_[nst++] = clock64(); } while (0)
+#else
+#define ZP_PSTAMP() do { } while (0)
+#endif
+
+// 1 / norm as 16-bit pieces for the matrix cores.  bf16 has fp32's exponent range: three pieces
+// carry all 24 mantissa bits.  fp16 does not: the pieces are taken of rn * 2^-x with x chosen per
+// block of 32 keys so that the block's largest value sits at the top of fp16's range, which leaves
+// 39 bits below it; the accumulator is rescaled where the block changes.
+template <typename T> struct RnScale;
+template <> struct RnScale<BF16> { static constexpr bool per_block = false; };
+template <> struct RnScale<F16> { static constexpr bool per_block = true; };
+
 template <typename T>
 __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
   static_assert(T::bytes == 2, "16-bit caches only");
   typedef typename Mfma16<T>::V frag_t;
   constexpr int PIECES = kDmax / 8;
   constexpr int KSB = kDmax / 16;
-  constexpr int PLANE = (kPageRows + 4) * ROWH;   // the page, then the three planes of the key sum
 
   extern __shared__ __align__(16) char smem[];
-  char* k_pl = smem;                                                          // raw keys
-  unsigned long long* l_corr = (unsigned long long*)(smem + PLANE);           // claimed from a row
+  char* k_pl = smem;                                   // raw keys
+  char* s_pl = smem + kPgBytes;                        // [4][kDmax] 16-bit: summed key as hi, mid, lo; zeros
+  char* rn_pl = s_pl + 4 * kDmax * 2;                  // [4][kPageRows] 16-bit: 1 / norm as hi, mid, lo; zeros
+  unsigned long long* l_corr = (unsigned long long*)(rn_pl + 4 * kPageRows * 2);   // claimed from a row
   float* l_sum = (float*)(l_corr + kPageRows);
-  float* l_rn = l_sum + kPageRows;                                            // 1 / norm
+  float* l_rn = l_sum + kPageRows;                     // 1 / norm
   int* l_col = (int*)(l_rn + kPageRows);
-  float* l_part = (float*)(l_col + kPageRows);     // [waves][kDmax] partial key sums
+  int* l_bexp = l_col + kPageRows;                     // [kPageWaves] scale exponent of a block's rn pieces
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int half = lane >> 5, col = lane & 31;
+#ifdef ZP_PAGE_STAMP
+  long long st_[10];
+  int nst = 0;
+  const long long wall0 = wall_clock64();
+#endif
+  ZP_PSTAMP();
   const int jp = blockIdx.x % p.NB;
   const int h = (blockIdx.x / p.NB) % p.Hkv;
   const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
@@ -1072,44 +1119,51 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
   if (rpid >= p.num_pages) rpid = -1;
   if (rpid < 0) {
     for (int s = tid; s < p.BS; s += kPageThreads) Elem<T>::st(p.r_out, obase + s, -INFINITY);
+#ifdef ZP_PAGE_STAMP
+    if (tid == 0 && blockIdx.x < kPageStampMax) zp_page_stamp_buf[(int64_t)blockIdx.x * 12 + 11] = -1;
+#endif
     return;
   }
   const int dpieces = p.D / 8;
-  const int64_t k_row = (int64_t)p.Hkv * p.D * 2;
+  const int k_row = p.Hkv * p.D * 2;
   const char* page = p.k + (l * p.k_sl + (int64_t)rpid * p.k_sp) * 2 + (int64_t)h * p.D * 2;
-
-  // ---- copy the page into LDS; the raw keys also stay in registers for the key sum
-  const int piece = tid % PIECES, row0 = tid / PIECES;       // 32 rows per iteration
-  constexpr int ROWS_PER_IT = kPageThreads / PIECES;
-  constexpr int ITERS = kPageRows / ROWS_PER_IT;
-  u32x4 raw[ITERS];
-#pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
-    const int row = it * ROWS_PER_IT + row0;
-    raw[it] = *(const u32x4*)(page + (int64_t)(row < p.BS ? row : 0) * k_row +
-                              (piece < dpieces ? piece : 0) * 16);
-  }
-  if (tid < kPageRows) { l_col[tid] = -1; l_corr[tid] = 0ull; }
-#pragma unroll
-  for (int it = 0; it < ITERS; ++it) {
-    const int row = it * ROWS_PER_IT + row0;
-    if (!(row < p.BS && piece < dpieces)) raw[it] = u32x4{0u, 0u, 0u, 0u};   // past the page / head dim: zeros
-    if (row < p.BS) *(u32x4*)(k_pl + row * ROWH + piece * 16) = raw[it];
-  }
-  __syncthreads();
-
-  // ---- norms from the diagonal of the Gram matrix: wave a multiplies its own block (a, a), which
-  // the claim rule needs anyway, and the 32 lanes that hold a diagonal entry turn it into 1 / norm
   const int nrb = p.BS / 32;
   const int a = wave;
+
+  if (dpieces < PIECES) {   // the tail of every key row must read as zero
+    for (int i = tid; i < kPgBytes / 4; i += kPageThreads) ((uint32_t*)k_pl)[i] = 0u;
+    __syncthreads();
+  }
+  // ---- the page into LDS: wave a requests row block a, eight instructions of four rows
+  if (wave < nrb) {
+    const int st_g = (lane >> 4) * 4 + (lane & 3), st_r = (lane >> 2) & 3;
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(page + (int64_t)a * 32 * k_row), 0, 32 * k_row, 0x00020000);
+    if (st_g < dpieces) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)(k_pl + (a * 8 + i) * kPgGrp), 16,
+                                                 st_r * k_row + st_g * 16, i * 4 * k_row, 0, 0);
+    }
+  }
+  if (tid < kPageRows) { l_col[tid] = -1; l_corr[tid] = 0ull; }
+  if (tid < kDmax / 2) ((uint32_t*)(s_pl + 3 * kDmax * 2))[tid] = 0u;
+  else if (tid < kDmax / 2 + kPageRows / 2) ((uint32_t*)(rn_pl + 3 * kPageRows * 2))[tid - kDmax / 2] = 0u;
+  ZP_PSTAMP();   // 1: page requested
+
+  // ---- norms from the diagonal of the Gram matrix: wave a multiplies its own block (a, a) as soon
+  // as its own rows have landed; the 32 lanes that hold a diagonal entry turn it into 1 / norm.
+  // Fragment of k-step s of this lane's row: base + (s / 2) * 256 + (s % 2) * 32.
+  const int rd_off = (col >> 2) * kPgGrp + (col & 3) * 64 + half * 16;
   frag_t ak[KSB];
   f32x16_t diag;
 #pragma unroll
   for (int r = 0; r < 16; ++r) diag[r] = 0.f;
   if (wave < nrb) {
-    const char* arow = k_pl + (a * 32 + col) * ROWH + half * 16;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    const char* arow = k_pl + a * 8 * kPgGrp + rd_off;
 #pragma unroll
-    for (int s = 0; s < KSB; ++s) ak[s] = *(const frag_t*)(arow + s * 32);
+    for (int s = 0; s < KSB; ++s) ak[s] = *(const frag_t*)(arow + (s >> 1) * 256 + (s & 1) * 32);
 #pragma unroll
     for (int s = 0; s < KSB; ++s) diag = Mfma16<T>::run(ak[s], ak[s], diag);
     // lane (col, half) owns rows (r/4)*8 + half*4 + r%4 of column col: entry (col, col) is its
@@ -1118,81 +1172,108 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
     float ss = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) ss = r == my_r ? diag[r] : ss;
+    const bool mine = ((col & 7) >> 2) == half;
     // the quotient only scales fp32 sums: the 1-ulp reciprocal is exact enough
     const float rn = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr));
-    if (((col & 7) >> 2) == half) {
+    float f = rn;
+    if constexpr (RnScale<T>::per_block) {
+      int e = mine ? (int)((__float_as_uint(rn) >> 23) & 0xffu) : 0;   // biased exponent
+      e = half_max_i(e);
+      e = max(e, lane_xor32(e));
+      const int x = e - 127 - 14;          // rn = f * 2^x, the block's largest f in [2^14, 2^15)
+      f = ldexpf(rn, -x);
+      if (lane == 0) l_bexp[a] = x;
+    }
+    if (mine) {
       l_rn[a * 32 + col] = rn;
       l_sum[a * 32 + col] = ss * rn * rn;      // |e_i|^2, taken off the row sum below
+      uint16_t o[3];
+      Split3<T>::run(f, o);
+#pragma unroll
+      for (int pl = 0; pl < 3; ++pl) *(uint16_t*)(rn_pl + pl * kPageRows * 2 + (a * 32 + col) * 2) = o[pl];
     }
   }
+  ZP_PSTAMP();   // 2: norms of wave 0's block
   __syncthreads();
+  ZP_PSTAMP();   // 3: page and norms complete
 
-  // ---- summed normalised key S = sum_j rn_j k_j (fp32, fixed order over the waves), stored as
-  // three 16-bit planes behind the page so that the matrix cores can multiply the keys with it
-  {
-    float cs[8];
+  // ---- summed normalised key S = sum_j rn_j k_j on the matrix cores, by the upper four waves
+  // (which have one tile fewer below): wave 7 - t takes the head dims 32 t .. 32 t + 31 and walks
+  // the keys sixteen at a time.  A: rows 0..2 = the pieces of rn (lanes col >= 3 read zeros);
+  // B: the keys transposed.  The three rows of the result are added smallest first and stored as
+  // three 16-bit planes, so that the matrix cores can multiply the keys with S as well.
+  if (wave >= kPageWaves - 4) {
+    const int dt = kPageWaves - 1 - wave;
+    f32x16_t acc;
 #pragma unroll
-    for (int q = 0; q < 8; ++q) cs[q] = 0.f;
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    const char* asrc = rn_pl + (col < 3 ? col : 3) * kPageRows * 2 + half * 16;
+    // transposing read: lane i of a group of sixteen supplies the address of key row i / 4, four
+    // dims at (i % 4) * 4 of the group's sixteen dims; groups: (half, dims 16 (g & 1) ..)
+    const int i16 = lane & 15, g4 = lane >> 4;
+    const char* bsrc = k_pl + (g4 >> 1) * 2 * kPgGrp + dt * 256 + (i16 >> 2) * 64 +
+                       ((g4 & 1) * 2 + ((i16 & 3) >> 1)) * 16 + (i16 & 1) * 8;
+    // a block of 32 keys is two k-steps; the operands of the next block are requested before the
+    // products of this one, so the chain of dependent products does not also wait for LDS
+    int xcur = 0;
+    frag_t af[2][2];
+    s16x4_t bl[2][2], bh[2][2];
+    auto fetch = [&](int blk, auto buf) {
 #pragma unroll
-    for (int it = 0; it < ITERS; ++it) {
-      const int row = it * ROWS_PER_IT + row0;
-      const float rn = row < p.BS ? l_rn[row] : 0.f;
-      float e[8];
-      Unpack<T>::run(vec16{raw[it].x, raw[it].y, raw[it].z, raw[it].w}, e);
+      for (int u = 0; u < 2; ++u) {
+        const int ks = 2 * blk + u;
+        af[buf.value][u] = *(const frag_t*)(asrc + ks * 32);
+        bl[buf.value][u] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (s16x4_t __attribute__((address_space(3)))*)(bsrc + ks * 4 * kPgGrp));
+        bh[buf.value][u] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (s16x4_t __attribute__((address_space(3)))*)(bsrc + (ks * 4 + 1) * kPgGrp));
+      }
+    };
+    auto products = [&](int blk, auto buf) {
+      if constexpr (RnScale<T>::per_block) {
+        const int xb = l_bexp[blk];
+        if (blk > 0) {
 #pragma unroll
-      for (int q = 0; q < 8; ++q) cs[q] = fmaf(e[q], rn, cs[q]);
+          for (int r = 0; r < 3; ++r) acc[r] = ldexpf(acc[r], xcur - xb);
+        }
+        xcur = xb;
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const s16x8_t bb = __builtin_shufflevector(bl[buf.value][u], bh[buf.value][u], 0, 1, 2, 3, 4, 5, 6, 7);
+        acc = Mfma16<T>::run(af[buf.value][u], __builtin_bit_cast(frag_t, bb), acc);
+      }
+    };
+    typedef std::integral_constant<int, 0> B0;
+    typedef std::integral_constant<int, 1> B1;
+    fetch(0, B0{});
+#pragma unroll 1
+    for (int blk = 0; blk < nrb; blk += 2) {
+      if (blk + 1 < nrb) fetch(blk + 1, B1{});
+      products(blk, B0{});
+      if (blk + 1 < nrb) {
+        if (blk + 2 < nrb) fetch(blk + 2, B0{});
+        products(blk + 1, B1{});
+      }
     }
-    // the four key rows a wave handles per iteration sit 16 lanes apart
+    if (half == 0) {
+      float sv = (acc[2] + acc[1]) + acc[0];
+      if constexpr (RnScale<T>::per_block) sv = ldexpf(sv, xcur);
+      uint16_t o[3];
+      Split3<T>::run(sv, o);
 #pragma unroll
-    for (int q = 0; q < 8; ++q) {
-      cs[q] += lane_xor16(cs[q]);
-      cs[q] += lane_xor32(cs[q]);
-    }
-    if (lane < PIECES) {
-      float* dst = l_part + wave * kDmax + piece * 8;
-      *(float4*)dst = make_float4(cs[0], cs[1], cs[2], cs[3]);
-      *(float4*)(dst + 4) = make_float4(cs[4], cs[5], cs[6], cs[7]);
+      for (int pl = 0; pl < 3; ++pl) *(uint16_t*)(s_pl + pl * kDmax * 2 + (dt * 32 + col) * 2) = o[pl];
     }
   }
-  __syncthreads();
-  if (tid < kDmax) {
-    float sv = 0.f;
-#pragma unroll
-    for (int w = 0; w < kPageWaves; ++w) sv += l_part[w * kDmax + tid];
-    uint16_t o[3];
-    Split3<T>::run(sv, o);
-#pragma unroll
-    for (int pl = 0; pl < 3; ++pl) *(uint16_t*)(k_pl + (kPageRows + pl) * ROWH + tid * 2) = o[pl];
-  }
-  __syncthreads();
+  ZP_PSTAMP();   // 4: (wave 0 has nothing to do for the key sum)
 
   // ---- Gram tiles: wave a owns row block a and the column blocks (a + d) mod n
+  float rn_row[16];
   if (wave < nrb) {
-    float rn_row[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) rn_row[r] = l_rn[a * 32 + (r >> 2) * 8 + half * 4 + (r & 3)];
-    // row sums without the matrix: sum_{j != i} e_i.e_j = rn_i (k_i . S) - |e_i|^2, the products
-    // k_i . S as one more tile whose columns 0..2 are the planes of S
-    {
-      f32x16_t acc;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-      const char* srow = k_pl + (kPageRows + (col < 3 ? col : 0)) * ROWH + half * 16;
-#pragma unroll
-      for (int s = 0; s < KSB; ++s) {
-        frag_t bk = *(const frag_t*)(srow + s * 32);
-        if (col >= 3) __builtin_memset(&bk, 0, sizeof(bk));
-        acc = Mfma16<T>::run(ak[s], bk, acc);
-      }
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        // lane col 0 adds the lo, mid and hi products (lanes col 2, 1, 0), smallest first
-        const float t = (dpp_row_shl<2>(acc[r]) + dpp_row_shl<1>(acc[r])) + acc[r];
-        if (col == 0) {
-          const int row = a * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-          l_sum[row] = t * rn_row[r] - l_sum[row];
-        }
-      }
+    for (int q = 0; q < 4; ++q) {   // the lane's rows come in runs of four
+      const float4 v = *(const float4*)(l_rn + a * 32 + q * 8 + half * 4);
+      rn_row[4 * q] = v.x; rn_row[4 * q + 1] = v.y; rn_row[4 * q + 2] = v.z; rn_row[4 * q + 3] = v.w;
     }
     // a tile whose largest entry stays below this cannot hold a claim (slack for the rounding of
     // the two ways the scale factors are multiplied in)
@@ -1205,7 +1286,7 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
     for (int d = 0; d < nd; ++d) {
       const int cb = a + d < nrb ? a + d : a + d - nrb;
       f32x16_t acc;
-      const char* brow = k_pl + (cb * 32 + col) * ROWH + half * 16;
+      const char* brow = k_pl + cb * 8 * kPgGrp + rd_off;
       const int cslot = cb * 32 + col;
       const float rn_col = l_rn[cslot];
       if (d == 0) {
@@ -1218,7 +1299,7 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
         frag_t bk[KSB];
 #pragma unroll
-        for (int s = 0; s < KSB; ++s) bk[s] = *(const frag_t*)(brow + s * 32);
+        for (int s = 0; s < KSB; ++s) bk[s] = *(const frag_t*)(brow + (s >> 1) * 256 + (s & 1) * 32);
 #pragma unroll
         for (int s = 0; s < KSB; ++s) acc = Mfma16<T>::run(ak[s], bk[s], acc);
       }
@@ -1256,34 +1337,88 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
       }
     }
   }
+  ZP_PSTAMP();   // 5: tiles of wave 0
   __syncthreads();
-  // ---- value of every key's claimed entry (16 lanes per key), subtracted from the row it was
-  // taken from.  Several keys may claim from one row: the values are added as 2^-32 fixed point
-  // with integer atomics, which is exact for a cosine above 2^-8 and does not depend on the order
-  // of the additions.
-  {
-    const int piece = tid % PIECES, g = tid / PIECES;
-#pragma unroll 1
-    for (int j = g; j < p.BS; j += kPageThreads / PIECES) {
-      const int c = l_col[j];
-      // c == j: with a negative threshold the zeroed diagonal entry itself can be the claim; its
-      // value is 0, nothing to hand back
-      if (c < 0 || c == j) continue;      // uniform over the 16 lanes of a key
-      const u32x4 kj = *(const u32x4*)(k_pl + j * ROWH + piece * 16);
-      const u32x4 kc = *(const u32x4*)(k_pl + c * ROWH + piece * 16);
-      float ej[8], ec[8];
-      Unpack<T>::run(vec16{kj.x, kj.y, kj.z, kj.w}, ej);
-      Unpack<T>::run(vec16{kc.x, kc.y, kc.z, kc.w}, ec);
-      float t = 0.f;
+  ZP_PSTAMP();   // 6: tiles of all waves, key sum planes
+
+  // ---- row sums without the matrix: sum_{j != i} e_i.e_j = rn_i (k_i . S) - |e_i|^2, the products
+  // k_i . S as one more tile whose columns 0..2 are the planes of S (the other lanes read zeros)
+  if (wave < nrb) {
+    f32x16_t acc;
 #pragma unroll
-      for (int q = 0; q < 8; ++q) t = fmaf(ej[q], ec[q], t);
-      t = pieces_sum<PIECES>(t);
-      if (piece == 0) atomicAdd(&l_corr[c], to_fixed32(t * (l_rn[j] * l_rn[c])));
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    const char* srow = s_pl + (col < 3 ? col : 3) * kDmax * 2 + half * 16;
+#pragma unroll
+    for (int s = 0; s < KSB; ++s) acc = Mfma16<T>::run(ak[s], *(const frag_t*)(srow + s * 32), acc);
+    float t[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r)   // lane col 0 adds the lo, mid and hi products (lanes col 2, 1, 0), smallest first
+      t[r] = (dpp_row_shl<2>(acc[r]) + dpp_row_shl<1>(acc[r])) + acc[r];
+    if (col == 0) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        float4* dst = (float4*)(l_sum + a * 32 + q * 8 + half * 4);
+        float4 v = *dst;
+        v.x = t[4 * q] * rn_row[4 * q] - v.x;
+        v.y = t[4 * q + 1] * rn_row[4 * q + 1] - v.y;
+        v.z = t[4 * q + 2] * rn_row[4 * q + 2] - v.z;
+        v.w = t[4 * q + 3] * rn_row[4 * q + 3] - v.w;
+        *dst = v;
+      }
     }
   }
+  // ---- value of every key's claimed entry, subtracted from the row it was taken from.  Several
+  // keys may claim from one row: the values are added as 2^-32 fixed point with integer atomics,
+  // which is exact for a cosine above 2^-8 and does not depend on the order of the additions.
+  // Wave w looks at the keys 32 w .. 32 w + 31 at once (most have no claim) and then handles the
+  // ones that have, four at a time with sixteen lanes per key.
+  {
+    static_assert(PIECES == 16, "sixteen lanes per key");
+    const int key = wave * 32 + col;
+    const int cl = key < p.BS ? l_col[key] : -1;
+    // cl == key: with a negative threshold the zeroed diagonal entry itself can be the claim; its
+    // value is 0, nothing to hand back
+    unsigned todo = (unsigned)__builtin_amdgcn_ballot_w64(half == 0 && cl >= 0 && cl != key);
+    const int q = lane >> 4, piece = lane & 15;
+    const int poff = (piece >> 2) * 256 + (piece & 3) * 16;
+    while (todo) {
+      unsigned m = todo;           // the q-th lowest key with a claim goes to lane group q
+#pragma unroll
+      for (int i = 0; i < 3; ++i) m = i < q ? m & (m - 1) : m;
+      const int jl = m ? __builtin_ctz(m) : -1;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) todo &= todo - 1;
+      const int c = __builtin_amdgcn_ds_bpermute((jl < 0 ? 0 : jl) << 2, cl);
+      if (jl >= 0) {               // uniform over the 16 lanes of a key
+        const int j = wave * 32 + jl;
+        const u32x4 kj = *(const u32x4*)(k_pl + (j >> 2) * kPgGrp + (j & 3) * 64 + poff);
+        const u32x4 kc = *(const u32x4*)(k_pl + (c >> 2) * kPgGrp + (c & 3) * 64 + poff);
+        float ej[8], ec[8];
+        Unpack<T>::run(vec16{kj.x, kj.y, kj.z, kj.w}, ej);
+        Unpack<T>::run(vec16{kc.x, kc.y, kc.z, kc.w}, ec);
+        float t = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t = fmaf(ej[e], ec[e], t);
+        t = pieces_sum<PIECES>(t);
+        if (piece == 0) atomicAdd(&l_corr[c], to_fixed32(t * (l_rn[j] * l_rn[c])));
+      }
+    }
+  }
+  ZP_PSTAMP();   // 7: row sums and claim values of wave 0
   __syncthreads();
+  ZP_PSTAMP();   // 8
   if (tid < p.BS) Elem<T>::st(p.r_out, obase + tid, l_sum[tid] - from_fixed32(l_corr[tid]));
+#ifdef ZP_PAGE_STAMP
+  ZP_PSTAMP();   // 9
+  if (tid == 0 && blockIdx.x < kPageStampMax) {
+    long long* dst = zp_page_stamp_buf + (int64_t)blockIdx.x * 12;
+    for (int i = 0; i < 10; ++i) dst[i] = i < nst ? st_[i] : 0;
+    dst[10] = wall0;
+    dst[11] = wall_clock64() - wall0;
+  }
+#endif
 }
+#undef ZP_PSTAMP
 
 // ------------------------------------------------------------------ raw, 16-bit caches
 // All-pairs variant over the whole sequence.  Four launches; the claims use the symmetric scheme
@@ -1951,8 +2086,8 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
   const size_t tail = (RAW ? 0 : (size_t)a.BS * 20) + sizeof(int) * 2 * a.NB;
   if constexpr (T::bytes == 2 && !RAW) {
     if (a.BS <= kPageRows && a.BS % 32 == 0) {
-      const size_t smem = (size_t)(kPageRows + 4) * ROWH + (size_t)kPageRows * 20 +
-                          (size_t)kPageWaves * kDmax * 4;
+      const size_t smem = (size_t)kPgBytes + 4 * kDmax * 2 + 4 * kPageRows * 2 +
+                          (size_t)kPageRows * 20 + sizeof(int) * kPageWaves;
       if (hipFuncSetAttribute((const void*)gram_page_kernel<T>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
         zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
