@@ -16,8 +16,11 @@
 //                      resident in LDS, one barrier, both operands read from that copy.
 //   gram_split_kernel  16-bit caches, lightning with pages above 256 keys: normalised keys
 //                      split into two bf16 planes, three MFMAs per k-step, full matrix.
-//   gram_page_kernel   16-bit caches, lightning: stored keys on the matrix cores, 1/norm
-//                      factors on the accumulators, every pair of key blocks once.
+//   gram_page_kernel   16-bit caches, lightning: a workgroup walks the pages of one (layer,
+//                      sequence, kv head) row; stored keys loaded straight into LDS and put on
+//                      the matrix cores, 1/norm factors on the accumulators, every pair of key
+//                      blocks once, the summed key as a product over the keys, the next page
+//                      requested while a page's row sums are finished.
 //   raw_prep_kernel, gram_raw_kernel, raw_claim_value_kernel, raw_chain_kernel
 //                      16-bit caches, raw: the same over the pages of a sequence, the row sums
 //                      accumulated in the cache dtype chunk by chunk as the reference does.
@@ -1052,7 +1055,9 @@ template <> struct Split3<F16> {
 //   * the summed normalised key  sum_j rn_j k_j  is a matrix product too, contracted over the
 //     keys: A = rn as three 16-bit pieces (rows 0..2), B = the keys read through the transposing
 //     LDS load (`ds_read_b64_tr_b16`: lane i of sixteen receives column i of a 4 x 16 block).
-// One plane of raw keys in LDS (65 KB), so two workgroups share a compute unit.
+// One plane of raw keys in LDS (65 KB), so two workgroups share a compute unit.  A workgroup
+// walks the pages of one row: once the tiles of a page are done nothing reads its keys in LDS
+// any more, so the next page is requested then and lands while the row sums are finished.
 constexpr int kPgGrp = 1040;                          // bytes from one group of four key rows to the next
 constexpr int kPgBytes = (kPageRows / 4) * kPgGrp;    // the page in LDS
 typedef short s16x4_t __attribute__((ext_vector_type(4)));
@@ -1081,7 +1086,7 @@ template <> struct RnScale<BF16> { static constexpr bool per_block = false; };
 template <> struct RnScale<F16> { static constexpr bool per_block = true; };
 
 template <typename T>
-__global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
+__global__ __launch_bounds__(kPageThreads, 4) void gram_page_kernel(GramArgs p) {
   static_assert(T::bytes == 2, "16-bit caches only");
   typedef typename Mfma16<T>::V frag_t;
   constexpr int PIECES = kDmax / 8;
@@ -1091,210 +1096,276 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
   char* k_pl = smem;                                   // raw keys
   char* s_pl = smem + kPgBytes;                        // [4][kDmax] 16-bit: summed key as hi, mid, lo; zeros
   char* rn_pl = s_pl + 4 * kDmax * 2;                  // [4][kPageRows] 16-bit: 1 / norm as hi, mid, lo; zeros
-  unsigned long long* l_corr = (unsigned long long*)(rn_pl + 4 * kPageRows * 2);   // claimed from a row
-  float* l_sum = (float*)(l_corr + kPageRows);
-  float* l_rn = l_sum + kPageRows;                     // 1 / norm
+  // claimed from a row / row sums: two copies, taken in turn by the pages of the walk, because a
+  // page's last phase reads them while the next page's first phase writes them
+  unsigned long long* l_corr2 = (unsigned long long*)(rn_pl + 4 * kPageRows * 2);
+  float* l_sum2 = (float*)(l_corr2 + 2 * kPageRows);
+  float* l_rn = l_sum2 + 2 * kPageRows;                // 1 / norm
   int* l_col = (int*)(l_rn + kPageRows);
   int* l_bexp = l_col + kPageRows;                     // [kPageWaves] scale exponent of a block's rn pieces
+  int* l_code = l_bexp + kPageWaves;                   // [NB] the block table row
 
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int half = lane >> 5, col = lane & 31;
+  const int tid = threadIdx.x;
 #ifdef ZP_PAGE_STAMP
   long long st_[10];
   int nst = 0;
-  const long long wall0 = wall_clock64();
 #endif
-  ZP_PSTAMP();
-  const int jp = blockIdx.x % p.NB;
-  const int h = (blockIdx.x / p.NB) % p.Hkv;
-  const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
-  const int l = blockIdx.x / (p.NB * p.Hkv * p.B);
+  // a workgroup walks the pages of one (layer, sequence, kv head) row
+  const int h = blockIdx.x % p.Hkv;
+  const int b = (blockIdx.x / p.Hkv) % p.B;
+  const int l = blockIdx.x / (p.Hkv * p.B);
   const int Tn = p.NB * p.BS;
-  const int64_t obase = (((int64_t)l * p.B + b) * p.Hkv + h) * Tn + (int64_t)jp * p.BS;
+  const int64_t rowbase = (((int64_t)l * p.B + b) * p.Hkv + h) * Tn;
   const float epsr = Elem<T>::rnd(p.eps);
-
-  const int code = p.table[(int64_t)b * p.NB + jp];
-  int rpid = page_is_pad(code) ? -1 : page_id(code);
-  if (rpid >= p.num_pages) rpid = -1;
-  if (rpid < 0) {
-    for (int s = tid; s < p.BS; s += kPageThreads) Elem<T>::st(p.r_out, obase + s, -INFINITY);
-#ifdef ZP_PAGE_STAMP
-    if (tid == 0 && blockIdx.x < kPageStampMax) zp_page_stamp_buf[(int64_t)blockIdx.x * 12 + 11] = -1;
-#endif
-    return;
-  }
   const int dpieces = p.D / 8;
   const int k_row = p.Hkv * p.D * 2;
-  const char* page = p.k + (l * p.k_sl + (int64_t)rpid * p.k_sp) * 2 + (int64_t)h * p.D * 2;
+  const char* layer = p.k + l * p.k_sl * 2 + (int64_t)h * p.D * 2;
   const int nrb = p.BS / 32;
-  const int a = wave;
 
+  for (int j = tid; j < p.NB; j += kPageThreads) l_code[j] = p.table[(int64_t)b * p.NB + j];
+  if (tid < kDmax / 2) ((uint32_t*)(s_pl + 3 * kDmax * 2))[tid] = 0u;
+  else if (tid < kDmax / 2 + kPageRows / 2) ((uint32_t*)(rn_pl + 3 * kPageRows * 2))[tid - kDmax / 2] = 0u;
   if (dpieces < PIECES) {   // the tail of every key row must read as zero
     for (int i = tid; i < kPgBytes / 4; i += kPageThreads) ((uint32_t*)k_pl)[i] = 0u;
-    __syncthreads();
   }
-  // ---- the page into LDS: wave a requests row block a, eight instructions of four rows
-  if (wave < nrb) {
-    const int st_g = (lane >> 4) * 4 + (lane & 3), st_r = (lane >> 2) & 3;
+  __syncthreads();
+  // page id of table entry j, or -1 (wave-uniform)
+  auto page_of = [&](int j) {
+    const int code = __builtin_amdgcn_readfirstlane(l_code[j]);
+    const int pid = page_is_pad(code) ? -1 : page_id(code);
+    return pid < p.num_pages ? pid : -1;
+  };
+  auto next_valid = [&](int j) {
+    while (j < p.NB && page_of(j) < 0) ++j;
+    return j;
+  };
+  for (int j = 0; j < p.NB; ++j) {      // entries without a page score -inf
+    if (page_of(j) >= 0) continue;
+    for (int s = tid; s < p.BS; s += kPageThreads) Elem<T>::st(p.r_out, rowbase + (int64_t)j * p.BS + s, -INFINITY);
+  }
+  // ---- a page into LDS: wave w requests row block w, eight instructions of four rows
+  auto request = [&](int j, int w, int ln) {
+    if (w >= nrb) return;
+    const int st_g = (ln >> 4) * 4 + (ln & 3), st_r = (ln >> 2) & 3;
+    const char* page = layer + (int64_t)page_of(j) * p.k_sp * 2;
     const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(page + (int64_t)a * 32 * k_row), 0, 32 * k_row, 0x00020000);
+        (void*)(page + (int64_t)w * 32 * k_row), 0, 32 * k_row, 0x00020000);
+    const int voff = st_r * k_row + st_g * 16;
     if (st_g < dpieces) {
 #pragma unroll
       for (int i = 0; i < 8; ++i)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)(k_pl + (a * 8 + i) * kPgGrp), 16,
-                                                 st_r * k_row + st_g * 16, i * 4 * k_row, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)(k_pl + (w * 8 + i) * kPgGrp), 16, voff,
+                                                 i * 4 * k_row, 0, 0);
     }
-  }
-  if (tid < kPageRows) { l_col[tid] = -1; l_corr[tid] = 0ull; }
-  if (tid < kDmax / 2) ((uint32_t*)(s_pl + 3 * kDmax * 2))[tid] = 0u;
-  else if (tid < kDmax / 2 + kPageRows / 2) ((uint32_t*)(rn_pl + 3 * kPageRows * 2))[tid - kDmax / 2] = 0u;
-  ZP_PSTAMP();   // 1: page requested
+  };
 
-  // ---- norms from the diagonal of the Gram matrix: wave a multiplies its own block (a, a) as soon
-  // as its own rows have landed; the 32 lanes that hold a diagonal entry turn it into 1 / norm.
-  // Fragment of k-step s of this lane's row: base + (s / 2) * 256 + (s % 2) * 32.
-  const int rd_off = (col >> 2) * kPgGrp + (col & 3) * 64 + half * 16;
-  frag_t ak[KSB];
-  f32x16_t diag;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) diag[r] = 0.f;
-  if (wave < nrb) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    const char* arow = k_pl + a * 8 * kPgGrp + rd_off;
-#pragma unroll
-    for (int s = 0; s < KSB; ++s) ak[s] = *(const frag_t*)(arow + (s >> 1) * 256 + (s & 1) * 32);
-#pragma unroll
-    for (int s = 0; s < KSB; ++s) diag = Mfma16<T>::run(ak[s], ak[s], diag);
-    // lane (col, half) owns rows (r/4)*8 + half*4 + r%4 of column col: entry (col, col) is its
-    // register (col/8)*4 + col%4 when (col%8)/4 == half
-    const int my_r = (col >> 3) * 4 + (col & 3);
-    float ss = 0.f;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) ss = r == my_r ? diag[r] : ss;
-    const bool mine = ((col & 7) >> 2) == half;
-    // the quotient only scales fp32 sums: the 1-ulp reciprocal is exact enough
-    const float rn = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr));
-    float f = rn;
-    if constexpr (RnScale<T>::per_block) {
-      int e = mine ? (int)((__float_as_uint(rn) >> 23) & 0xffu) : 0;   // biased exponent
-      e = half_max_i(e);
-      e = max(e, lane_xor32(e));
-      const int x = e - 127 - 14;          // rn = f * 2^x, the block's largest f in [2^14, 2^15)
-      f = ldexpf(rn, -x);
-      if (lane == 0) l_bexp[a] = x;
-    }
-    if (mine) {
-      l_rn[a * 32 + col] = rn;
-      l_sum[a * 32 + col] = ss * rn * rn;      // |e_i|^2, taken off the row sum below
-      uint16_t o[3];
-      Split3<T>::run(f, o);
-#pragma unroll
-      for (int pl = 0; pl < 3; ++pl) *(uint16_t*)(rn_pl + pl * kPageRows * 2 + (a * 32 + col) * 2) = o[pl];
-    }
-  }
-  ZP_PSTAMP();   // 2: norms of wave 0's block
-  __syncthreads();
-  ZP_PSTAMP();   // 3: page and norms complete
+  int jp = next_valid(0);
+  if (jp < p.NB) request(jp, __builtin_amdgcn_readfirstlane(tid >> 6), tid & 63);
+  int par = 0;
+#pragma unroll 1
+  while (jp < p.NB) {
+    // Lane and wave numbers are made opaque once per page: what is derived from them (LDS
+    // addresses, row indices) is then computed where a page uses it instead of once before the
+    // loop and held in registers through all of it, which the tiles have none to spare for.
+    int lane = tid & 63;
+    asm volatile("" : "+v"(lane));
+    int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    asm volatile("" : "+s"(wave));
+    const int half = lane >> 5, col = lane & 31;
+    const int a = wave;
+    // fragment of k-step s of this lane's row: base + (s / 2) * 256 + (s % 2) * 32
+    const int rd_off = (col >> 2) * kPgGrp + (col & 3) * 64 + half * 16;
+#ifdef ZP_PAGE_STAMP
+    nst = 0;
+    const long long wall0 = wall_clock64();
+#endif
+    ZP_PSTAMP();
+    unsigned long long* l_corr = l_corr2 + par * kPageRows;
+    float* l_sum = l_sum2 + par * kPageRows;
+    const char* page = layer + (int64_t)page_of(jp) * p.k_sp * 2;
+    const int64_t obase = rowbase + (int64_t)jp * p.BS;
+    const int tix = wave * 64 + lane;
+    if (tix < kPageRows) { l_col[tix] = -1; l_corr[tix] = 0ull; }
+    ZP_PSTAMP();   // 1
 
-  // ---- summed normalised key S = sum_j rn_j k_j on the matrix cores, by the upper four waves
-  // (which have one tile fewer below): wave 7 - t takes the head dims 32 t .. 32 t + 31 and walks
-  // the keys sixteen at a time.  A: rows 0..2 = the pieces of rn (lanes col >= 3 read zeros);
-  // B: the keys transposed.  The three rows of the result are added smallest first and stored as
-  // three 16-bit planes, so that the matrix cores can multiply the keys with S as well.
-  if (wave >= kPageWaves - 4) {
-    const int dt = kPageWaves - 1 - wave;
-    f32x16_t acc;
+    // ---- norms from the diagonal of the Gram matrix: wave a multiplies its own block (a, a) as
+    // soon as its own rows have landed; the 32 lanes that hold a diagonal entry turn it into 1 / norm
+    frag_t ak[KSB];
+    f32x16_t diag;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-    const char* asrc = rn_pl + (col < 3 ? col : 3) * kPageRows * 2 + half * 16;
-    // transposing read: lane i of a group of sixteen supplies the address of key row i / 4, four
-    // dims at (i % 4) * 4 of the group's sixteen dims; groups: (half, dims 16 (g & 1) ..)
-    const int i16 = lane & 15, g4 = lane >> 4;
-    const char* bsrc = k_pl + (g4 >> 1) * 2 * kPgGrp + dt * 256 + (i16 >> 2) * 64 +
-                       ((g4 & 1) * 2 + ((i16 & 3) >> 1)) * 16 + (i16 & 1) * 8;
-    // a block of 32 keys is two k-steps; the operands of the next block are requested before the
-    // products of this one, so the chain of dependent products does not also wait for LDS
-    int xcur = 0;
-    frag_t af[2][2];
-    s16x4_t bl[2][2], bh[2][2];
-    auto fetch = [&](int blk, auto buf) {
+    for (int r = 0; r < 16; ++r) diag[r] = 0.f;
+    if (wave < nrb) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      const char* arow = k_pl + a * 8 * kPgGrp + rd_off;
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const int ks = 2 * blk + u;
-        af[buf.value][u] = *(const frag_t*)(asrc + ks * 32);
-        bl[buf.value][u] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (s16x4_t __attribute__((address_space(3)))*)(bsrc + ks * 4 * kPgGrp));
-        bh[buf.value][u] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (s16x4_t __attribute__((address_space(3)))*)(bsrc + (ks * 4 + 1) * kPgGrp));
-      }
-    };
-    auto products = [&](int blk, auto buf) {
+      for (int s = 0; s < KSB; ++s) ak[s] = *(const frag_t*)(arow + (s >> 1) * 256 + (s & 1) * 32);
+#pragma unroll
+      for (int s = 0; s < KSB; ++s) diag = Mfma16<T>::run(ak[s], ak[s], diag);
+      // lane (col, half) owns rows (r/4)*8 + half*4 + r%4 of column col: entry (col, col) is its
+      // register (col/8)*4 + col%4 when (col%8)/4 == half
+      const int my_r = (col >> 3) * 4 + (col & 3);
+      float ss = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) ss = r == my_r ? diag[r] : ss;
+      const bool mine = ((col & 7) >> 2) == half;
+      // the quotient only scales fp32 sums: the 1-ulp reciprocal is exact enough
+      const float rn = __builtin_amdgcn_rcpf(fmaxf(Elem<T>::rnd(sqrtf(ss)), epsr));
+      float f = rn;
       if constexpr (RnScale<T>::per_block) {
-        const int xb = l_bexp[blk];
-        if (blk > 0) {
-#pragma unroll
-          for (int r = 0; r < 3; ++r) acc[r] = ldexpf(acc[r], xcur - xb);
-        }
-        xcur = xb;
+        int e = mine ? (int)((__float_as_uint(rn) >> 23) & 0xffu) : 0;   // biased exponent
+        e = half_max_i(e);
+        e = max(e, lane_xor32(e));
+        const int x = e - 127 - 14;          // rn = f * 2^x, the block's largest f in [2^14, 2^15)
+        f = ldexpf(rn, -x);
+        if (lane == 0) l_bexp[a] = x;
       }
+      if (mine) {
+        l_rn[a * 32 + col] = rn;
+        l_sum[a * 32 + col] = ss * rn * rn;      // |e_i|^2, taken off the row sum below
+        uint16_t o[3];
+        Split3<T>::run(f, o);
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        const s16x8_t bb = __builtin_shufflevector(bl[buf.value][u], bh[buf.value][u], 0, 1, 2, 3, 4, 5, 6, 7);
-        acc = Mfma16<T>::run(af[buf.value][u], __builtin_bit_cast(frag_t, bb), acc);
-      }
-    };
-    typedef std::integral_constant<int, 0> B0;
-    typedef std::integral_constant<int, 1> B1;
-    fetch(0, B0{});
-#pragma unroll 1
-    for (int blk = 0; blk < nrb; blk += 2) {
-      if (blk + 1 < nrb) fetch(blk + 1, B1{});
-      products(blk, B0{});
-      if (blk + 1 < nrb) {
-        if (blk + 2 < nrb) fetch(blk + 2, B0{});
-        products(blk + 1, B1{});
+        for (int pl = 0; pl < 3; ++pl) *(uint16_t*)(rn_pl + pl * kPageRows * 2 + (a * 32 + col) * 2) = o[pl];
       }
     }
-    if (half == 0) {
-      float sv = (acc[2] + acc[1]) + acc[0];
-      if constexpr (RnScale<T>::per_block) sv = ldexpf(sv, xcur);
-      uint16_t o[3];
-      Split3<T>::run(sv, o);
-#pragma unroll
-      for (int pl = 0; pl < 3; ++pl) *(uint16_t*)(s_pl + pl * kDmax * 2 + (dt * 32 + col) * 2) = o[pl];
-    }
-  }
-  ZP_PSTAMP();   // 4: (wave 0 has nothing to do for the key sum)
+    ZP_PSTAMP();   // 2: norms of wave 0's block
+    __syncthreads();
+    ZP_PSTAMP();   // 3: page and norms complete
 
-  // ---- Gram tiles: wave a owns row block a and the column blocks (a + d) mod n
-  float rn_row[16];
-  if (wave < nrb) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {   // the lane's rows come in runs of four
-      const float4 v = *(const float4*)(l_rn + a * 32 + q * 8 + half * 4);
-      rn_row[4 * q] = v.x; rn_row[4 * q + 1] = v.y; rn_row[4 * q + 2] = v.z; rn_row[4 * q + 3] = v.w;
-    }
-    // a tile whose largest entry stays below this cannot hold a claim (slack for the rounding of
-    // the two ways the scale factors are multiplied in)
-    const float thr_lo = p.threshold - fabsf(p.threshold) * 1e-5f - 1e-30f;
-    int dcol[16];
-#pragma unroll
-    for (int r = 0; r < 16; ++r) dcol[r] = -1;
-    const int nd = nrb / 2 + ((nrb & 1) || a < nrb / 2 ? 1 : 0);   // distances 0 .. nd-1
-#pragma unroll 1
-    for (int d = 0; d < nd; ++d) {
-      const int cb = a + d < nrb ? a + d : a + d - nrb;
+    // ---- summed normalised key S = sum_j rn_j k_j on the matrix cores, by the upper four waves
+    // (which have one tile fewer below): wave 7 - t takes the head dims 32 t .. 32 t + 31 and walks
+    // the keys sixteen at a time.  A: rows 0..2 = the pieces of rn (lanes col >= 3 read zeros);
+    // B: the keys transposed.  The three rows of the result are added smallest first and stored as
+    // three 16-bit planes, so that the matrix cores can multiply the keys with S as well.
+    if (wave >= kPageWaves - 4) {
+      const int dt = kPageWaves - 1 - wave;
       f32x16_t acc;
-      const char* brow = k_pl + cb * 8 * kPgGrp + rd_off;
-      const int cslot = cb * 32 + col;
-      const float rn_col = l_rn[cslot];
-      if (d == 0) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+      const char* asrc = rn_pl + (col < 3 ? col : 3) * kPageRows * 2 + half * 16;
+      // transposing read: lane i of a group of sixteen supplies the address of key row i / 4, four
+      // dims at (i % 4) * 4 of the group's sixteen dims; groups: (half, dims 16 (g & 1) ..)
+      const int i16 = lane & 15, g4 = lane >> 4;
+      const char* bsrc = k_pl + (g4 >> 1) * 2 * kPgGrp + dt * 256 + (i16 >> 2) * 64 +
+                         ((g4 & 1) * 2 + ((i16 & 3) >> 1)) * 16 + (i16 & 1) * 8;
+      // a block of 32 keys is two k-steps; the operands of the next block are requested before the
+      // products of this one, so the chain of dependent products does not also wait for LDS
+      int xcur = 0;
+      frag_t af[2][2];
+      s16x4_t bl[2][2], bh[2][2];
+      auto fetch = [&](int blk, auto buf) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const int ks = 2 * blk + u;
+          af[buf.value][u] = *(const frag_t*)(asrc + ks * 32);
+          bl[buf.value][u] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (s16x4_t __attribute__((address_space(3)))*)(bsrc + ks * 4 * kPgGrp));
+          bh[buf.value][u] = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+              (s16x4_t __attribute__((address_space(3)))*)(bsrc + (ks * 4 + 1) * kPgGrp));
+        }
+      };
+      auto products = [&](int blk, auto buf) {
+        if constexpr (RnScale<T>::per_block) {
+          const int xb = l_bexp[blk];
+          if (blk > 0) {
+#pragma unroll
+            for (int r = 0; r < 3; ++r) acc[r] = ldexpf(acc[r], xcur - xb);
+          }
+          xcur = xb;
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const s16x8_t bb = __builtin_shufflevector(bl[buf.value][u], bh[buf.value][u], 0, 1, 2, 3, 4, 5, 6, 7);
+          acc = Mfma16<T>::run(af[buf.value][u], __builtin_bit_cast(frag_t, bb), acc);
+        }
+      };
+      typedef std::integral_constant<int, 0> B0;
+      typedef std::integral_constant<int, 1> B1;
+      fetch(0, B0{});
+#pragma unroll 1
+      for (int blk = 0; blk < nrb; blk += 2) {
+        if (blk + 1 < nrb) fetch(blk + 1, B1{});
+        products(blk, B0{});
+        if (blk + 1 < nrb) {
+          if (blk + 2 < nrb) fetch(blk + 2, B0{});
+          products(blk + 1, B1{});
+        }
+      }
+      if (half == 0) {
+        float sv = (acc[2] + acc[1]) + acc[0];
+        if constexpr (RnScale<T>::per_block) sv = ldexpf(sv, xcur);
+        uint16_t o[3];
+        Split3<T>::run(sv, o);
+#pragma unroll
+        for (int pl = 0; pl < 3; ++pl) *(uint16_t*)(s_pl + pl * kDmax * 2 + (dt * 32 + col) * 2) = o[pl];
+      }
+    }
+    ZP_PSTAMP();   // 4: (wave 0 has nothing to do for the key sum)
+
+    // ---- Gram tiles: wave a owns row block a and the column blocks (a + d) mod n
+    float rn_row[16];
+    if (wave < nrb) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {   // the lane's rows come in runs of four
+        const float4 v = *(const float4*)(l_rn + a * 32 + q * 8 + half * 4);
+        rn_row[4 * q] = v.x; rn_row[4 * q + 1] = v.y; rn_row[4 * q + 2] = v.z; rn_row[4 * q + 3] = v.w;
+      }
+      // a tile whose largest entry stays below this cannot hold a claim (slack for the rounding of
+      // the two ways the scale factors are multiplied in)
+      const float thr_lo = p.threshold - fabsf(p.threshold) * 1e-5f - 1e-30f;
+      float rn_max = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) rn_max = fmaxf(rn_max, rn_row[r]);
+      int dcol[16];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) dcol[r] = -1;
+      const int nd = nrb / 2 + ((nrb & 1) || a < nrb / 2 ? 1 : 0);   // distances 0 .. nd-1
+      // what a tile feeds: the last column over the threshold of the keys on both of its sides
+      auto scan = [&](const f32x16_t& acc, int cb, bool off_diagonal) {
+        const int cslot = cb * 32 + col;
+        const float rn_col = l_rn[cslot];
+        // most tiles hold no entry over the threshold, and one maximum decides.  With a positive
+        // threshold only positive products matter, and those are at most the largest product
+        // times the largest row factor: that bound needs no multiplication per entry.
+        if (thr_lo > 0.f) {
+          float amax = 0.f;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) amax = fmaxf(amax, acc[r]);
+          if (!__any(amax * rn_max * rn_col > thr_lo)) return;
+        }
+        float big = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) big = fmaxf(big, acc[r] * rn_row[r]);
+        if (!__any(big * rn_col > thr_lo)) return;
+        // row side: key (a, r) sees column cslot; column side (off the diagonal block, where both
+        // (i, j) and (j, i) are computed): key cslot sees the rows of block a, whose index grows
+        // with r inside a lane, so the last hit is the largest
+        int rlast = -1;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const bool over = acc[r] * (rn_row[r] * rn_col) > p.threshold;
+          dcol[r] = max(dcol[r], over ? cslot : -1);
+          rlast = over ? r : rlast;
+        }
+        if (off_diagonal && __any(rlast >= 0)) {
+          int ci = rlast < 0 ? -1 : a * 32 + (rlast >> 2) * 8 + half * 4 + (rlast & 3);
+          ci = max(ci, lane_xor32(ci));
+          if (half == 0 && ci >= 0) atomicMax(&l_col[cslot], ci);
+        }
+      };
+      {
         // the diagonal block was multiplied for the norms; a key against itself counts as 0
+        f32x16_t acc;
 #pragma unroll
         for (int r = 0; r < 16; ++r)
           acc[r] = (r >> 2) * 8 + half * 4 + (r & 3) == col ? 0.f : diag[r];
-      } else {
+        scan(acc, a, false);
+      }
+#pragma unroll 1
+      for (int d = 1; d < nd; ++d) {
+        const int cb = a + d < nrb ? a + d : a + d - nrb;
+        const char* brow = k_pl + cb * 8 * kPgGrp + rd_off;
+        f32x16_t acc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
         frag_t bk[KSB];
@@ -1302,121 +1373,112 @@ __global__ __launch_bounds__(kPageThreads) void gram_page_kernel(GramArgs p) {
         for (int s = 0; s < KSB; ++s) bk[s] = *(const frag_t*)(brow + (s >> 1) * 256 + (s & 1) * 32);
 #pragma unroll
         for (int s = 0; s < KSB; ++s) acc = Mfma16<T>::run(ak[s], bk[s], acc);
+        scan(acc, cb, true);
       }
-      // most tiles hold no entry over the threshold: one maximum decides
-      float big = -INFINITY;
+      // most waves see no entry over the threshold: then the reduction over the lanes is skipped
+      bool mine = false;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) big = fmaxf(big, acc[r] * rn_row[r]);
-      if (!__any(big * rn_col > thr_lo)) continue;
-      // row side: key (a, r) sees column cslot; column side (off the diagonal block, where both
-      // (i, j) and (j, i) are computed): key cslot sees the rows of block a, whose index grows
-      // with r inside a lane, so the last hit is the largest
-      int rlast = -1;
+      for (int r = 0; r < 16; ++r) mine |= dcol[r] >= 0;
+      if (__any(mine)) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const bool over = acc[r] * (rn_row[r] * rn_col) > p.threshold;
-        dcol[r] = max(dcol[r], over ? cslot : -1);
-        rlast = over ? r : rlast;
-      }
-      if (d != 0 && __any(rlast >= 0)) {
-        int ci = rlast < 0 ? -1 : a * 32 + (rlast >> 2) * 8 + half * 4 + (rlast & 3);
-        ci = max(ci, lane_xor32(ci));
-        if (half == 0 && ci >= 0) atomicMax(&l_col[cslot], ci);
+        for (int r = 0; r < 16; ++r) {
+          const int c = half_max_i(dcol[r]);
+          if (col == 0 && c >= 0)
+            atomicMax(&l_col[a * 32 + (r >> 2) * 8 + half * 4 + (r & 3)], c);
+        }
       }
     }
-    // most waves see no entry over the threshold: then the reduction over the lanes is skipped
-    bool mine = false;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) mine |= dcol[r] >= 0;
-    if (__any(mine)) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int c = half_max_i(dcol[r]);
-        if (col == 0 && c >= 0)
-          atomicMax(&l_col[a * 32 + (r >> 2) * 8 + half * 4 + (r & 3)], c);
-      }
-    }
-  }
-  ZP_PSTAMP();   // 5: tiles of wave 0
-  __syncthreads();
-  ZP_PSTAMP();   // 6: tiles of all waves, key sum planes
+    ZP_PSTAMP();   // 5: tiles of wave 0
+    __syncthreads();
+    ZP_PSTAMP();   // 6: tiles of all waves, key sum planes
 
-  // ---- row sums without the matrix: sum_{j != i} e_i.e_j = rn_i (k_i . S) - |e_i|^2, the products
-  // k_i . S as one more tile whose columns 0..2 are the planes of S (the other lanes read zeros)
-  if (wave < nrb) {
-    f32x16_t acc;
+    // ---- nothing below reads the page in LDS: the next page of the row is requested now and
+    // lands while this one finishes
+    const int nj = next_valid(jp + 1);
+    if (nj < p.NB) request(nj, wave, lane);
+
+    // ---- row sums without the matrix: sum_{j != i} e_i.e_j = rn_i (k_i . S) - |e_i|^2, the products
+    // k_i . S as one more tile whose columns 0..2 are the planes of S (the other lanes read zeros)
+    if (wave < nrb) {
+      f32x16_t acc;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-    const char* srow = s_pl + (col < 3 ? col : 3) * kDmax * 2 + half * 16;
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+      const char* srow = s_pl + (col < 3 ? col : 3) * kDmax * 2 + half * 16;
 #pragma unroll
-    for (int s = 0; s < KSB; ++s) acc = Mfma16<T>::run(ak[s], *(const frag_t*)(srow + s * 32), acc);
-    float t[16];
+      for (int s = 0; s < KSB; ++s) acc = Mfma16<T>::run(ak[s], *(const frag_t*)(srow + s * 32), acc);
+      float t[16];
 #pragma unroll
-    for (int r = 0; r < 16; ++r)   // lane col 0 adds the lo, mid and hi products (lanes col 2, 1, 0), smallest first
-      t[r] = (dpp_row_shl<2>(acc[r]) + dpp_row_shl<1>(acc[r])) + acc[r];
-    if (col == 0) {
+      for (int r = 0; r < 16; ++r)   // lane col 0 adds the lo, mid and hi products (lanes col 2, 1, 0), smallest first
+        t[r] = (dpp_row_shl<2>(acc[r]) + dpp_row_shl<1>(acc[r])) + acc[r];
+      if (col == 0) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        float4* dst = (float4*)(l_sum + a * 32 + q * 8 + half * 4);
-        float4 v = *dst;
-        v.x = t[4 * q] * rn_row[4 * q] - v.x;
-        v.y = t[4 * q + 1] * rn_row[4 * q + 1] - v.y;
-        v.z = t[4 * q + 2] * rn_row[4 * q + 2] - v.z;
-        v.w = t[4 * q + 3] * rn_row[4 * q + 3] - v.w;
-        *dst = v;
+        for (int q = 0; q < 4; ++q) {
+          float4* dst = (float4*)(l_sum + a * 32 + q * 8 + half * 4);
+          float4 v = *dst;
+          v.x = t[4 * q] * rn_row[4 * q] - v.x;
+          v.y = t[4 * q + 1] * rn_row[4 * q + 1] - v.y;
+          v.z = t[4 * q + 2] * rn_row[4 * q + 2] - v.z;
+          v.w = t[4 * q + 3] * rn_row[4 * q + 3] - v.w;
+          *dst = v;
+        }
       }
     }
-  }
-  // ---- value of every key's claimed entry, subtracted from the row it was taken from.  Several
-  // keys may claim from one row: the values are added as 2^-32 fixed point with integer atomics,
-  // which is exact for a cosine above 2^-8 and does not depend on the order of the additions.
-  // Wave w looks at the keys 32 w .. 32 w + 31 at once (most have no claim) and then handles the
-  // ones that have, four at a time with sixteen lanes per key.
-  {
-    static_assert(PIECES == 16, "sixteen lanes per key");
-    const int key = wave * 32 + col;
-    const int cl = key < p.BS ? l_col[key] : -1;
-    // cl == key: with a negative threshold the zeroed diagonal entry itself can be the claim; its
-    // value is 0, nothing to hand back
-    unsigned todo = (unsigned)__builtin_amdgcn_ballot_w64(half == 0 && cl >= 0 && cl != key);
-    const int q = lane >> 4, piece = lane & 15;
-    const int poff = (piece >> 2) * 256 + (piece & 3) * 16;
-    while (todo) {
-      unsigned m = todo;           // the q-th lowest key with a claim goes to lane group q
+    // ---- value of every key's claimed entry, subtracted from the row it was taken from.  Several
+    // keys may claim from one row: the values are added as 2^-32 fixed point with integer atomics,
+    // which is exact for a cosine above 2^-8 and does not depend on the order of the additions.
+    // Wave w looks at the keys 32 w .. 32 w + 31 at once (most have no claim) and then handles the
+    // ones that have, four at a time with sixteen lanes per key; the two key rows come from
+    // global memory (the cache: the page was read a moment ago).
+    {
+      static_assert(PIECES == 16, "sixteen lanes per key");
+      const int key = wave * 32 + col;
+      const int cl = key < p.BS ? l_col[key] : -1;
+      // cl == key: with a negative threshold the zeroed diagonal entry itself can be the claim; its
+      // value is 0, nothing to hand back
+      unsigned todo = (unsigned)__builtin_amdgcn_ballot_w64(half == 0 && cl >= 0 && cl != key);
+      const int q = lane >> 4, piece = lane & 15;
+      while (todo) {
+        unsigned m = todo;           // the q-th lowest key with a claim goes to lane group q
 #pragma unroll
-      for (int i = 0; i < 3; ++i) m = i < q ? m & (m - 1) : m;
-      const int jl = m ? __builtin_ctz(m) : -1;
+        for (int i = 0; i < 3; ++i) m = i < q ? m & (m - 1) : m;
+        const int jl = m ? __builtin_ctz(m) : -1;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) todo &= todo - 1;
-      const int c = __builtin_amdgcn_ds_bpermute((jl < 0 ? 0 : jl) << 2, cl);
-      if (jl >= 0) {               // uniform over the 16 lanes of a key
-        const int j = wave * 32 + jl;
-        const u32x4 kj = *(const u32x4*)(k_pl + (j >> 2) * kPgGrp + (j & 3) * 64 + poff);
-        const u32x4 kc = *(const u32x4*)(k_pl + (c >> 2) * kPgGrp + (c & 3) * 64 + poff);
-        float ej[8], ec[8];
-        Unpack<T>::run(vec16{kj.x, kj.y, kj.z, kj.w}, ej);
-        Unpack<T>::run(vec16{kc.x, kc.y, kc.z, kc.w}, ec);
-        float t = 0.f;
+        for (int i = 0; i < 4; ++i) todo &= todo - 1;
+        const int c = __builtin_amdgcn_ds_bpermute((jl < 0 ? 0 : jl) << 2, cl);
+        if (jl >= 0) {               // uniform over the 16 lanes of a key
+          const int j = wave * 32 + jl;
+          u32x4 kj = u32x4{0u, 0u, 0u, 0u}, kc = kj;
+          if (piece < dpieces) {
+            kj = *(const u32x4*)(page + (int64_t)j * k_row + piece * 16);
+            kc = *(const u32x4*)(page + (int64_t)c * k_row + piece * 16);
+          }
+          float ej[8], ec[8];
+          Unpack<T>::run(vec16{kj.x, kj.y, kj.z, kj.w}, ej);
+          Unpack<T>::run(vec16{kc.x, kc.y, kc.z, kc.w}, ec);
+          float t = 0.f;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) t = fmaf(ej[e], ec[e], t);
-        t = pieces_sum<PIECES>(t);
-        if (piece == 0) atomicAdd(&l_corr[c], to_fixed32(t * (l_rn[j] * l_rn[c])));
+          for (int e = 0; e < 8; ++e) t = fmaf(ej[e], ec[e], t);
+          t = pieces_sum<PIECES>(t);
+          if (piece == 0) atomicAdd(&l_corr[c], to_fixed32(t * (l_rn[j] * l_rn[c])));
+        }
       }
     }
-  }
-  ZP_PSTAMP();   // 7: row sums and claim values of wave 0
-  __syncthreads();
-  ZP_PSTAMP();   // 8
-  if (tid < p.BS) Elem<T>::st(p.r_out, obase + tid, l_sum[tid] - from_fixed32(l_corr[tid]));
+    ZP_PSTAMP();   // 7: row sums and claim values of wave 0
+    __syncthreads();
+    ZP_PSTAMP();   // 8
+    if (tix < p.BS) Elem<T>::st(p.r_out, obase + tix, l_sum[tix] - from_fixed32(l_corr[tix]));
 #ifdef ZP_PAGE_STAMP
-  ZP_PSTAMP();   // 9
-  if (tid == 0 && blockIdx.x < kPageStampMax) {
-    long long* dst = zp_page_stamp_buf + (int64_t)blockIdx.x * 12;
-    for (int i = 0; i < 10; ++i) dst[i] = i < nst ? st_[i] : 0;
-    dst[10] = wall0;
-    dst[11] = wall_clock64() - wall0;
-  }
+    ZP_PSTAMP();   // 9
+    if (tid == 0 && blockIdx.x * p.NB + jp < kPageStampMax) {
+      long long* dst = zp_page_stamp_buf + ((int64_t)blockIdx.x * p.NB + jp) * 12;
+      for (int i = 0; i < 10; ++i) dst[i] = i < nst ? st_[i] : 0;
+      dst[10] = wall0;
+      dst[11] = wall_clock64() - wall0;
+    }
 #endif
+    jp = nj;
+    par ^= 1;
+  }
 }
 #undef ZP_PSTAMP
 
@@ -2085,9 +2147,11 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
   dim3 grid((unsigned)((int64_t)L * a.B * a.Hkv * a.NB));
   const size_t tail = (RAW ? 0 : (size_t)a.BS * 20) + sizeof(int) * 2 * a.NB;
   if constexpr (T::bytes == 2 && !RAW) {
-    if (a.BS <= kPageRows && a.BS % 32 == 0) {
-      const size_t smem = (size_t)kPgBytes + 4 * kDmax * 2 + 4 * kPageRows * 2 +
-                          (size_t)kPageRows * 20 + sizeof(int) * kPageWaves;
+    // one workgroup per (layer, sequence, kv head) row; the block table row sits in LDS
+    const size_t smem = (size_t)kPgBytes + 4 * kDmax * 2 + 4 * kPageRows * 2 +
+                        (size_t)kPageRows * (2 * 8 + 2 * 4 + 4 + 4) + sizeof(int) * (kPageWaves + a.NB);
+    if (a.BS <= kPageRows && a.BS % 32 == 0 && smem <= 80 * 1024) {
+      grid = dim3((unsigned)((int64_t)L * a.B * a.Hkv));
       if (hipFuncSetAttribute((const void*)gram_page_kernel<T>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
         zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
