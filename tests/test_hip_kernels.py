@@ -436,6 +436,29 @@ def test_redundancy_key_magnitudes(dev, dtype, scale, variant):
     _ulp_close(gr, wr, dtype, ulps=4)
 
 
+@pytest.mark.parametrize("dtype,span", [(torch.float16, 6), (torch.bfloat16, 14)])
+def test_lightning_redundancy_mixed_key_magnitudes(dev, dtype, span):
+    """Every key of a page scaled by its own power of two: the cosines do not change, and the page
+    kernel, which sums the keys weighted by 1 / norm on the matrix cores (fp16: in pieces scaled
+    per block of 32 keys), must not lose the small weights beside the large ones."""
+    from zipage_amd import kernel as K
+    s = _setup(97, dtype, L=1, B=2, Hkv=2, Hq=2, BS=256, nb_choices=(2, 3), budget=1, num_pages=10)
+    g = torch.Generator().manual_seed(13)
+    base = torch.randn((1, 1, 1, 2, 128), generator=g)
+    k0 = s["k"].float() * 0.7 + base
+    expo = torch.randint(-span, span + 1, k0.shape[:-1] + (1,), generator=g).float()
+    kw = dict(threshold=0.45, temperature=0.4, return_logits=True)
+    # the unscaled keys rounded first, so that scaling by a power of two is exact in both dtypes
+    k = (k0.to(dtype).float() * torch.exp2(expo)).to(dtype)
+    wl, wr = O.lightning_redudancy_score(k, s["enc"], **kw)
+    gl, gr = K.lightning_redudancy_score(k.to(dev), s["enc"].to(dev), **kw)
+    _ulp_close(gl, wl, dtype, ulps=1, abs_floor=1e-2)
+    _ulp_close(gr, wr, dtype, ulps=4)
+    # and the same scores as the unscaled keys give (the oracle's own invariance, then ours)
+    ul, _ = K.lightning_redudancy_score(k0.to(dtype).to(dev), s["enc"].to(dev), **kw)
+    _ulp_close(gl, ul.cpu(), dtype, ulps=2, abs_floor=1e-2)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("BS,D", [(128, 128), (512, 128), (256, 64), (64, 32), (192, 128)])
 @pytest.mark.parametrize("variant", ["lightning", "raw"])
