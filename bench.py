@@ -233,14 +233,30 @@ def run_pipeline(config, args, sw="pooling", batch=None, steps=None, warmup=None
 
     slices = wl.L if layers > 1 else 1
     sc = wl.score_cache
+    # Redundancy scores depend on the keys: a step that found the survivors of the last page still
+    # in that page would meet more duplicated keys with every step.  The one-layer workloads with
+    # a redundancy stage therefore take a fresh last page per step, as a decode refills it.
+    rot = None
+    if layers == 1 and cfg.use_redudancy:
+        from zipage_amd.bench.workload import fresh_last_pages
+        rot = fresh_last_pages(wl, 64)
+        desc += (" [every step finds fresh keys in each sequence's last page: 64 tables in turn]"
+                 if rot is not None else
+                 " [the pool has no spare pages for fresh last pages: the steps re-compress the "
+                 "same pages and meet keys duplicated by earlier steps]")
+    calls = [0]
 
     def step(timer=None):
+        tables, targets = wl.block_tables, wl.targets
+        if rot is not None:
+            tables, targets = rot[0][calls[0] % 64], rot[1][calls[0] % 64]
+            calls[0] += 1
         for i in range(layers):
             l = i % slices
             compress_layers(wl.k[l:l + 1] if layers > 1 else wl.k, wl.v[l:l + 1] if layers > 1 else wl.v,
                             wl.q[l:l + 1] if layers > 1 else wl.q,
                             sc if sc is None or layers == 1 else sc[l:l + 1], wl.query_ids,
-                            wl.block_tables, wl.compressed, wl.targets, cfg, timer=timer,
+                            tables, wl.compressed, targets, cfg, timer=timer,
                             fused_select=not args.separate_select_stages)
 
     for _ in range(warmup):

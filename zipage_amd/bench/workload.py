@@ -131,6 +131,47 @@ def ragged_batch(B, *, L=1, pool_pages=20000, budget=8, W=32, BS=256, dtype=torc
         budget=budget, W=W, tables=tables, placement=placement)
 
 
+def fresh_last_pages(wl: Workload, n: int, seed: int = 7):
+    """``n`` block tables (and target tables) for ``wl`` that differ in every sequence's LAST page:
+    table 0 is the workload's own, the others name pool pages nobody uses, filled with fresh
+    random keys, values and cached scores.  A benchmark that compresses the same sequences step
+    after step takes them in turn, as a decode would have refilled the last page between two
+    compressions; with one table the survivors copied out of the last page would also still sit in
+    it, and the redundancy kernels would meet more and more duplicated keys.
+    Returns ``(tables (n, B, NB) int32, targets (n, B, budget+1) int32)`` on the device, or ``None``
+    when the pool has fewer than ``(n - 1) * B`` spare pages."""
+    L, pool_pages = wl.k.shape[0], wl.k.shape[1]
+    dev = wl.k.device
+    used = {p for t in wl.tables for p in t} | set(wl.targets.flatten().tolist())
+    spare = [p for p in range(pool_pages) if p not in used]
+    B = wl.B
+    if n < 2 or len(spare) < (n - 1) * B:
+        return None
+    g = torch.Generator().manual_seed(seed)
+    order = torch.randperm(len(spare), generator=g)[:(n - 1) * B].tolist()
+    alt = [spare[i] for i in order]
+    idx = torch.tensor(alt, device=dev)
+    gg = torch.Generator(device=dev).manual_seed(seed)
+    for l in range(L):
+        for pool in (wl.k, wl.v):
+            pool[l, idx] = torch.randn((len(alt),) + tuple(pool.shape[2:]), generator=gg, device=dev,
+                                       dtype=torch.float32).to(pool.dtype)
+        if wl.score_cache is not None:
+            wl.score_cache[l, idx] = torch.rand((len(alt),) + tuple(wl.score_cache.shape[2:]),
+                                                generator=gg, device=dev).to(wl.score_cache.dtype)
+    targets0 = wl.targets.tolist()
+    tabs, tgts = [wl.block_tables], [wl.targets]
+    for i in range(n - 1):
+        tables, targets = [], []
+        for b in range(B):
+            last, new = wl.tables[b][-1], alt[i * B + b]
+            tables.append(list(wl.tables[b][:-1]) + [new])
+            targets.append([new if p == last else p for p in targets0[b]])
+        tabs.append(encode_tables(tables, dev))
+        tgts.append(torch.tensor(targets, dtype=torch.int32, device=dev))
+    return torch.stack(tabs), torch.stack(tgts)
+
+
 def algorithmic_bytes(wl: Workload, cfg, layers=None) -> dict:
     """HBM bytes each stage has to move for this workload (per launch over ``layers`` layers, all
     of the workload's by default):
