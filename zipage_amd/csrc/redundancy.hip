@@ -1238,6 +1238,9 @@ __global__ __launch_bounds__(kPageThreads, 4) void gram_page_kernel(GramArgs p) 
     // B: the keys transposed.  The three rows of the result are added smallest first and stored as
     // three 16-bit planes, so that the matrix cores can multiply the keys with S as well.
     if (wave >= kPageWaves - 4) {
+      // these four waves carry the key sum on top of their tiles and are what the barrier behind
+      // the tiles waits for: they issue ahead of the other waves of the compute unit until then
+      __builtin_amdgcn_s_setprio(2);
       const int dt = kPageWaves - 1 - wave;
       f32x16_t acc;
 #pragma unroll
@@ -1389,6 +1392,7 @@ __global__ __launch_bounds__(kPageThreads, 4) void gram_page_kernel(GramArgs p) 
       }
     }
     ZP_PSTAMP();   // 5: tiles of wave 0
+    __builtin_amdgcn_s_setprio(0);
     __syncthreads();
     ZP_PSTAMP();   // 6: tiles of all waves, key sum planes
 
