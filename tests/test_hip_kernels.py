@@ -485,6 +485,28 @@ def test_redundancy_page_and_head_sizes(dev, dtype, BS, D, variant):
         _ulp_close(gr, wr, dtype, ulps=4)
 
 
+@pytest.mark.parametrize("dtype,BS", [(torch.bfloat16, 64), (torch.float16, 128), (torch.float16, 256)])
+def test_lightning_redundancy_long_ragged_tables(dev, dtype, BS):
+    """Rows of 1 to 70 pages in one padded table (more entries than a wave has lanes): the page
+    kernel walks a row's pages one after the other and skips the padding."""
+    from zipage_amd.kernel import lightning_redudancy_score
+    perm = torch.randperm(120, generator=torch.Generator().manual_seed(101)).tolist()
+    tables, pos = [], 0
+    for nb in (9, 70, 1, 33):
+        tables.append(perm[pos:pos + nb])
+        pos += nb
+    enc = O.encode_block_table(tables)
+    assert enc.shape == (4, 70) and (enc == -1).any()
+    k = cases.make_caches(101, 1, 120, BS, 2, 2, 128, 32, 4, dtype, touched=cases.touched_pages(enc))[0]
+    base = torch.randn((1, 1, 1, 2, 128), generator=torch.Generator().manual_seed(3))
+    k = (k.float() * 0.7 + base).to(dtype)
+    kw = dict(threshold=0.45, temperature=0.4, return_logits=True)
+    wl, wr = O.lightning_redudancy_score(k, enc, **kw)
+    gl, gr = lightning_redudancy_score(k.to(dev), enc.to(dev), **kw)
+    _ulp_close(gl, wl, dtype, ulps=1, abs_floor=1e-2)
+    _ulp_close(gr, wr, dtype, ulps=4)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("nb_choices", [(1, 2), (3, 4), (5, 6), (7,)])
 def test_raw_redundancy_page_counts(dev, dtype, nb_choices):
