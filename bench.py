@@ -176,12 +176,12 @@ def run_pipeline(config, args, sw="pooling", batch=None, steps=None, warmup=None
     elif config == 3:
         from zipage_amd.bench.workload import QWEN3_0_6B
         batch, layers = batch or 128, 1
-        wl = ragged_batch(batch, L=1, pool_pages=2048, budget=8, W=32, seed=0, lengths=(2304, 2304),
+        wl = ragged_batch(batch, L=1, pool_pages=20000, budget=8, W=32, seed=0, lengths=(2304, 2304),
                           dtype=torch.float32, shape=QWEN3_0_6B, name="cfg3", with_score_cache=True,
                           compressed=True, place_tries=args.place_tries,
                           one_allocation=args.place_tries <= 1)
         desc = (f"configs[2]: {batch} sequences, 1 layer, Qwen3-0.6B attention shape (16q/8kv heads, "
-                "head_dim 128), fp32, 9 pages x 256 tokens, window 32, 2048-page pool, score -> global "
+                "head_dim 128), fp32, 9 pages x 256 tokens, window 32, 20k-page pool, score -> global "
                 "score (U(0,1) carried, decay 0.9, added) -> avg-pool 7 -> minus 0.5 x "
                 + ("raw all-pairs" if sw == "raw" else "lightning (same-page)")
                 + " redundancy (lambda 2/3) -> top-2048/head -> compact to 8 pages")
