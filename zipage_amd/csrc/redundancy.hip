@@ -1775,6 +1775,236 @@ void gram_raw_kernel(GramArgs p) {
   }
 }
 
+// The same for pages that are whole 128-key tiles, built like the page kernel of the lightning
+// variant: four waves, each with TWO row blocks of the row page in registers (64 rows), so a B
+// fragment read from LDS feeds two products; the column tiles go from global memory straight into
+// LDS (wave w requests rows 32 w .. 32 w + 31 of a tile, the layout of `gram_page_kernel`), two
+// buffers, one barrier per tile, the request for tile t + 1 under the products of tile t.  Two
+// workgroups per compute unit (two waves per SIMD, 256 registers each).
+constexpr int kRawTile = 128;
+constexpr int kRawTileBytes = (kRawTile / 4) * kPgGrp;
+template <typename T>
+__global__ __launch_bounds__(256, 2) void gram_raw_wide_kernel(GramArgs p) {
+  static_assert(T::bytes == 2, "16-bit caches only");
+  typedef typename Mfma16<T>::V frag_t;
+  constexpr int kThreads = 256, kWaves = 4, TNc = kRawTile;
+  constexpr int PIECES = kDmax / 8;
+  constexpr int NSUB = TNc / 32;
+  constexpr int KSB = kDmax / 16;
+
+  extern __shared__ __align__(16) char smem[];
+  char* buf0 = smem;                                // raw keys of a column tile
+  char* buf1 = smem + kRawTileBytes;
+  float* l_rn = (float*)(smem + 2 * kRawTileBytes); // [2][TNc] 1 / norm of the tile's keys
+  int* l_cside = (int*)(l_rn + 2 * TNc);            // [2][TNc] column-side claims of a tile
+  float* l_rnrow = (float*)(l_cside + 2 * TNc);     // [BS] 1 / norm of the row page's keys
+  int* vpage = (int*)(l_rnrow + p.BS);
+  int* vidx = vpage + p.NB;
+  __shared__ int nvalid_s, mine_s;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5, col = lane & 31;
+  const int jp = blockIdx.x % p.NB;
+  const int h = (blockIdx.x / p.NB) % p.Hkv;
+  const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
+  const int l = blockIdx.x / (p.NB * p.Hkv * p.B);
+  const int Tn = p.NB * p.BS;
+  const int64_t obase = (((int64_t)l * p.B + b) * p.Hkv + h) * Tn;
+
+  const int code = p.table[(int64_t)b * p.NB + jp];
+  int rpid = page_is_pad(code) ? -1 : page_id(code);
+  if (rpid >= p.num_pages) rpid = -1;
+  if (rpid < 0) return;
+  if (tid == 0) {
+    int n = 0, me = 0;
+    for (int j = 0; j < p.NB; ++j) {
+      const int c = p.table[(int64_t)b * p.NB + j];
+      const int pid = page_is_pad(c) ? -1 : page_id(c);
+      if (pid >= 0 && pid < p.num_pages) {
+        if (j == jp) me = n;
+        vpage[n] = pid; vidx[n] = j; ++n;
+      }
+    }
+    nvalid_s = n;
+    mine_s = me;
+  }
+  const int dpieces = p.D / 8;
+  if (dpieces < PIECES) {   // head dims below 128 leave the upper pieces of every LDS row at zero
+    for (int i = tid; i < 2 * kRawTileBytes / 4; i += kThreads) ((uint32_t*)smem)[i] = 0u;
+  }
+  if (tid < 2 * TNc) l_cside[tid] = -1;
+  for (int i = tid; i < p.BS; i += kThreads) l_rnrow[i] = p.ws_val[obase + (int64_t)jp * p.BS + i];
+  __syncthreads();
+  const int nv = nvalid_s, ia = mine_s;
+  const int nd = nv / 2 + (((nv & 1) || ia < nv / 2) ? 1 : 0);   // page distances 0 .. nd-1
+  const int tiles_per_page = p.BS / TNc;
+  const int ntiles = nd * tiles_per_page;
+  const int k_row = p.Hkv * p.D * 2;
+  const char* kbase = p.k + (l * p.k_sl) * 2 + (int64_t)h * p.D * 2;
+  const float* rn_all = p.ws_val + obase;           // written by raw_prep_kernel
+
+  auto tile_page = [&](int tile, int& d, int& toff) {
+    d = tile / tiles_per_page;
+    toff = (tile - d * tiles_per_page) * TNc;
+    const int ic = ia + d;
+    return ic < nv ? ic : ic - nv;
+  };
+  // tile -> LDS: eight instructions of four rows per wave; 1 / norm of the tile's keys to a register
+  const int st_g = (lane >> 4) * 4 + (lane & 3), st_r = (lane >> 2) & 3;
+  const int st_voff = st_r * k_row + st_g * 16;
+  float pre_rn = 0.f;
+  auto request = [&](int tile, char* buf) {
+    int d, toff;
+    const int ic = tile_page(tile, d, toff);
+    const int pid = __builtin_amdgcn_readfirstlane(vpage[ic]);
+    const char* src = kbase + (int64_t)pid * p.k_sp * 2 + (int64_t)(toff + wave * 32) * k_row;
+    const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, 32 * k_row, 0x00020000);
+    if (st_g < dpieces) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_ptr_t)(buf + (wave * 8 + i) * kPgGrp), 16, st_voff,
+                                                 i * 4 * k_row, 0, 0);
+    }
+    if (tid < TNc) pre_rn = rn_all[vidx[ic] * p.BS + toff + tid];
+  };
+  // Hands the column-side claims of a finished tile to the keys of its page and clears the slot.
+  auto flush_cside = [&](int tile) {
+    if (tid < TNc) {
+      int d, toff;
+      const int ic = tile_page(tile, d, toff);
+      int* slot = l_cside + (tile & 1) * TNc + tid;
+      const int v = *slot;
+      if (v >= 0) {
+        atomicMax(p.ws_col + obase + (int64_t)vidx[ic] * p.BS + toff + tid, v);
+        *slot = -1;
+      }
+    }
+  };
+  const float thr_lo = p.threshold - fabsf(p.threshold) * 1e-5f - 1e-30f;
+  // fragment of k-step s of this lane's row of a 32-row block: base + (s / 2) * 256 + (s % 2) * 32
+  const int rd_off = (col >> 2) * kPgGrp + (col & 3) * 64 + half * 16;
+
+  const int row_blocks = p.BS / 32;
+  const int NR = (row_blocks + 2 * kWaves - 1) / (2 * kWaves);
+  for (int rr = 0; rr < NR; ++rr) {
+    const int rb0 = (rr * kWaves + wave) * 2;          // this wave's two row blocks: rb0, rb0 + 1
+    const bool act0 = rb0 < row_blocks, act1 = rb0 + 1 < row_blocks;
+    // ---- A fragments: this lane's two key rows as stored; lane (row, half) holds k = 16 s + 8 half + i
+    frag_t ak0[KSB], ak1[KSB];
+    {
+      const char* src0 = kbase + (int64_t)rpid * p.k_sp * 2 + (int64_t)((act0 ? rb0 : 0) * 32 + col) * k_row;
+      const char* src1 = kbase + (int64_t)rpid * p.k_sp * 2 + (int64_t)((act1 ? rb0 + 1 : 0) * 32 + col) * k_row;
+#pragma unroll
+      for (int s = 0; s < KSB; ++s) {
+        const int pc = 2 * s + half;
+        u32x4 v0 = u32x4{0u, 0u, 0u, 0u}, v1 = v0;
+        if (pc < dpieces) {
+          v0 = *(const u32x4*)(src0 + pc * 16);
+          v1 = *(const u32x4*)(src1 + pc * 16);
+        }
+        ak0[s] = __builtin_bit_cast(frag_t, v0);
+        ak1[s] = __builtin_bit_cast(frag_t, v1);
+      }
+    }
+    float rn_row0[16], rn_row1[16];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const float4 v0 = *(const float4*)(l_rnrow + (act0 ? rb0 : 0) * 32 + half * 4 + g * 8);
+      const float4 v1 = *(const float4*)(l_rnrow + (act1 ? rb0 + 1 : 0) * 32 + half * 4 + g * 8);
+      rn_row0[4 * g] = v0.x; rn_row0[4 * g + 1] = v0.y; rn_row0[4 * g + 2] = v0.z; rn_row0[4 * g + 3] = v0.w;
+      rn_row1[4 * g] = v1.x; rn_row1[4 * g + 1] = v1.y; rn_row1[4 * g + 2] = v1.z; rn_row1[4 * g + 3] = v1.w;
+    }
+    int dcol0[16], dcol1[16];
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { dcol0[r] = -1; dcol1[r] = -1; }
+
+    if (ntiles > 0) request(0, buf0);
+    for (int tile = 0; tile < ntiles; ++tile) {
+      char* cur = (tile & 1) ? buf1 : buf0;
+      char* nxt = (tile & 1) ? buf0 : buf1;
+      // this wave's share of the tile (and its A fragments, the first time) has landed; after the
+      // barrier so has everybody's, and everybody is done with the tile before
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (tid < TNc) l_rn[(tile & 1) * TNc + tid] = pre_rn;
+      __syncthreads();
+      if (tile + 1 < ntiles) request(tile + 1, nxt);
+      if (tile > 0) flush_cside(tile - 1);   // its slot is next written two tiles from now
+      int d, toff;
+      const int ic = tile_page(tile, d, toff);
+      const int jc = vidx[ic];
+      // what a tile of 32 x 32 products feeds: the last column over the threshold of its rows and
+      // (other pages only: inside a page both (i, j) and (j, i) are computed) the last row over
+      // the threshold of its columns
+      auto scan = [&](f32x16_t& acc, int rb, const float* rn_row, int* dcol, int st, float rn_col) {
+        const int cslot = toff + st * 32 + col;
+        const int cidx = jc * p.BS + cslot;
+        if (d == 0) {
+          // the page against itself: a key against itself counts as 0
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3) == cslot) acc[r] = 0.f;
+        }
+        // most tiles hold no entry over the threshold: one maximum decides
+        float big = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) big = fmaxf(big, acc[r] * rn_row[r]);
+        if (!__any(big * rn_col > thr_lo)) return;
+        int rlast = -1;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const bool over = acc[r] * (rn_row[r] * rn_col) > p.threshold;
+          dcol[r] = max(dcol[r], over ? cidx : -1);
+          rlast = over ? r : rlast;
+        }
+        if (d != 0 && __any(rlast >= 0)) {
+          int ci = rlast < 0 ? -1 : jp * p.BS + rb * 32 + (rlast >> 2) * 8 + half * 4 + (rlast & 3);
+          ci = max(ci, lane_xor32(ci));
+          if (half == 0 && ci >= 0) atomicMax(&l_cside[(tile & 1) * TNc + st * 32 + col], ci);
+        }
+      };
+      if (act0) {
+#pragma unroll 1
+        for (int st = 0; st < NSUB; ++st) {
+          f32x16_t acc0, acc1;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
+          const char* brow = cur + st * 8 * kPgGrp + rd_off;
+          const float rn_col = l_rn[(tile & 1) * TNc + st * 32 + col];
+#pragma unroll
+          for (int s0 = 0; s0 < KSB; s0 += 4) {
+            frag_t bk[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) bk[s] = *(const frag_t*)(brow + ((s0 + s) >> 1) * 256 + ((s0 + s) & 1) * 32);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+              acc0 = Mfma16<T>::run(ak0[s0 + s], bk[s], acc0);
+              acc1 = Mfma16<T>::run(ak1[s0 + s], bk[s], acc1);
+            }
+          }
+          scan(acc0, rb0, rn_row0, dcol0, st, rn_col);
+          if (act1) scan(acc1, rb0 + 1, rn_row1, dcol1, st, rn_col);
+        }
+      }
+    }
+    __syncthreads();   // everybody is done with the last tile
+    if (ntiles > 0) flush_cside(ntiles - 1);
+    bool any_mine = false;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) any_mine |= dcol0[r] >= 0 || dcol1[r] >= 0;
+    if (__any(any_mine)) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int c0 = half_max_i(dcol0[r]), c1 = half_max_i(dcol1[r]);
+        const int64_t row = obase + (int64_t)jp * p.BS + rb0 * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+        if (act0 && col == 0 && c0 >= 0) atomicMax(p.ws_col + row, c0);
+        if (act1 && col == 0 && c1 >= 0) atomicMax(p.ws_col + row + 32, c1);
+      }
+    }
+    __syncthreads();   // the claim slots are clear again before the next round writes them
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(kThreads) void raw_claim_value_kernel(GramArgs p) {
   static_assert(T::bytes == 2, "16-bit caches only");
@@ -2201,20 +2431,26 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
     const size_t smem1 = 2 * (size_t)tn * ROWH + sizeof(int) * 4 * tn + sizeof(float) * a.BS +
                          sizeof(int) * 2 * a.NB;
     const void* fn = tn == 128 ? (const void*)gram_raw_kernel<T, 128> : (const void*)gram_raw_kernel<T, TN>;
+    // whole 128-key tiles: the four-wave kernel with two row blocks per wave
+    const size_t smemw = 2 * (size_t)kRawTileBytes + sizeof(int) * 4 * kRawTile + sizeof(float) * a.BS +
+                         sizeof(int) * 2 * a.NB;
+    const bool wide = tn == 128 && smemw <= 80 * 1024;
     const size_t smem2 = 3 * 32 * (size_t)ROWH + sizeof(int) * 32 * 256 + sizeof(int) * 2 * a.NB +
                          (size_t)a.NB * a.BS * 8;   // + the round's claim list
     if (smem2 > 160 * 1024) {
       zp_set_error("redundancy: a row of %d tokens exceeds LDS", a.NB * a.BS);
       return ZP_EUNSUPPORTED;
     }
-    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem1) != hipSuccess ||
+    if (hipFuncSetAttribute(wide ? (const void*)gram_raw_wide_kernel<T> : fn,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)(wide ? smemw : smem1)) != hipSuccess ||
         hipFuncSetAttribute((const void*)raw_chain_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize,
                             (int)smem2) != hipSuccess) {
       zp_set_error("redundancy: cannot reserve %zu / %zu bytes of LDS", smem1, smem2);
       return ZP_EHIP;
     }
     hipLaunchKernelGGL((raw_prep_kernel<T>), grid, dim3(kThreads), 0, st, a);
-    if (tn == 128) hipLaunchKernelGGL((gram_raw_kernel<T, 128>), grid, dim3(512), smem1, st, a);
+    if (wide) hipLaunchKernelGGL((gram_raw_wide_kernel<T>), grid, dim3(256), smemw, st, a);
+    else if (tn == 128) hipLaunchKernelGGL((gram_raw_kernel<T, 128>), grid, dim3(512), smem1, st, a);
     else hipLaunchKernelGGL((gram_raw_kernel<T, TN>), grid, dim3(512), smem1, st, a);
     hipLaunchKernelGGL((raw_claim_value_kernel<T>), grid, dim3(kThreads), 0, st, a);
     hipLaunchKernelGGL((raw_chain_kernel<T>), grid, dim3(512), smem2, st, a);
