@@ -38,6 +38,37 @@ template <int PIECES> __device__ __forceinline__ float pieces_sum(float v) {
   if (PIECES == 32) v += lane_xor16(v);
   return v;
 }
+// The valid pages of one block-table row in table order, listed in LDS by the first wave of the
+// workgroup (64 entries per step: one load per lane, a ballot ranks the valid ones), instead of a
+// serial walk by one thread with a global load per entry.  vpage[n] / vidx[n]: page id / table
+// index of the n-th valid page; vord[j]: rank of table entry j or -1; *n_out: their number; *me_out:
+// the rank of entry `jp` (0 when it is not valid).  Null pointers are skipped; the caller meets at
+// a barrier before reading.
+__device__ __forceinline__ void list_valid_pages(const int32_t* __restrict__ row, int NB, int num_pages,
+                                                 int jp, int* vpage, int* vidx, int* vord, int* n_out,
+                                                 int* me_out) {
+  if (threadIdx.x >= 64) return;
+  const int lane = threadIdx.x;
+  int n = 0;
+  if (lane == 0 && me_out) *me_out = 0;
+  for (int j0 = 0; j0 < NB; j0 += 64) {
+    const int j = j0 + lane;
+    const int c = j < NB ? row[j] : -1;
+    const int pid = page_is_pad(c) ? -1 : page_id(c);
+    const bool ok = pid >= 0 && pid < num_pages;
+    const unsigned long long m = __builtin_amdgcn_ballot_w64(ok);
+    const int pos = n + __builtin_popcountll(m & lanemask_lt());
+    if (ok) {
+      if (vpage) vpage[pos] = pid;
+      if (vidx) vidx[pos] = j;
+      if (me_out && j == jp) *me_out = pos;
+    }
+    if (vord && j < NB) vord[j] = ok ? pos : -1;
+    n += __builtin_popcountll(m);
+  }
+  if (lane == 0) *n_out = n;
+}
+
 // Over the 32 lanes of a wave half: the entry with the largest column index (and its value).
 __device__ __forceinline__ void last_claim_reduce(int& c, float& v) {
 #define ZP_CLAIM_STEP(OC, OV)              \
@@ -160,18 +191,10 @@ __global__ __launch_bounds__(NW * 64) void gram_kernel(GramArgs p) {
   }
 
   __shared__ int ncols_s;
-  if (tid == 0) {
-    int n = 0;
-    if (RAW) {
-      for (int j = 0; j < p.NB; ++j) {
-        const int c = p.table[(int64_t)b * p.NB + j];
-        const int pid = page_is_pad(c) ? -1 : page_id(c);
-        if (pid >= 0 && pid < p.num_pages) { vpage[n] = pid; vidx[n] = j; ++n; }
-      }
-    } else {
-      vpage[0] = rpid; vidx[0] = jp; n = 1;
-    }
-    ncols_s = n;
+  if (RAW) {
+    list_valid_pages(p.table + (int64_t)b * p.NB, p.NB, p.num_pages, jp, vpage, vidx, nullptr, &ncols_s, nullptr);
+  } else if (tid == 0) {
+    vpage[0] = rpid; vidx[0] = jp; ncols_s = 1;
   }
   for (int i = tid; i < 2 * TN * ROWF; i += kThreads) kbuf0[i] = 0.f;
   __syncthreads();
@@ -394,18 +417,7 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
   if (rpid < 0) return;
 
   __shared__ int nvalid_s, mine_s;
-  if (tid == 0) {
-    int n = 0, me = 0;
-    for (int j = 0; j < p.NB; ++j) {
-      const int c = p.table[(int64_t)b * p.NB + j];
-      const int pid = page_is_pad(c) ? -1 : page_id(c);
-      if (pid >= 0 && pid < p.num_pages) {
-        if (j == jp) me = n;
-        vpage[n] = pid; vidx[n] = j; ++n;
-      }
-    }
-    nvalid_s = n; mine_s = me;
-  }
+  list_valid_pages(p.table + (int64_t)b * p.NB, p.NB, p.num_pages, jp, vpage, vidx, nullptr, &nvalid_s, &mine_s);
   for (int i = tid; i < 2 * TN * ROWF; i += kThreads) kbuf0[i] = 0.f;
   __syncthreads();
   const int n = nvalid_s, ai = mine_s;
@@ -788,18 +800,10 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void gram_split_kernel(Gr
     return;
   }
   __shared__ int ncols_s;
-  if (tid == 0) {
-    int n = 0;
-    if (RAW) {
-      for (int j = 0; j < p.NB; ++j) {
-        const int c = p.table[(int64_t)b * p.NB + j];
-        const int pid = page_is_pad(c) ? -1 : page_id(c);
-        if (pid >= 0 && pid < p.num_pages) { vpage[n] = pid; vidx[n] = j; ++n; }
-      }
-    } else {
-      vpage[0] = rpid; vidx[0] = jp; n = 1;
-    }
-    ncols_s = n;
+  if (RAW) {
+    list_valid_pages(p.table + (int64_t)b * p.NB, p.NB, p.num_pages, jp, vpage, vidx, nullptr, &ncols_s, nullptr);
+  } else if (tid == 0) {
+    vpage[0] = rpid; vidx[0] = jp; ncols_s = 1;
   }
   for (int i = tid; i < 4 * PLANE / 4; i += kThreads) ((uint32_t*)smem)[i] = 0u;
   __syncthreads();
@@ -1600,19 +1604,7 @@ void gram_raw_kernel(GramArgs p) {
   int rpid = page_is_pad(code) ? -1 : page_id(code);
   if (rpid >= p.num_pages) rpid = -1;
   if (rpid < 0) return;
-  if (tid == 0) {
-    int n = 0, me = 0;
-    for (int j = 0; j < p.NB; ++j) {
-      const int c = p.table[(int64_t)b * p.NB + j];
-      const int pid = page_is_pad(c) ? -1 : page_id(c);
-      if (pid >= 0 && pid < p.num_pages) {
-        if (j == jp) me = n;
-        vpage[n] = pid; vidx[n] = j; ++n;
-      }
-    }
-    nvalid_s = n;
-    mine_s = me;
-  }
+  list_valid_pages(p.table + (int64_t)b * p.NB, p.NB, p.num_pages, jp, vpage, vidx, nullptr, &nvalid_s, &mine_s);
   // head dims below 128 leave the upper pieces of every LDS row at zero
   for (int i = tid; i < 2 * PLANE / 4; i += kThreads) ((uint32_t*)smem)[i] = 0u;
   if (tid < 2 * TNc) l_cside[tid] = -1;
@@ -1816,19 +1808,7 @@ __global__ __launch_bounds__(256, 2) void gram_raw_wide_kernel(GramArgs p) {
   int rpid = page_is_pad(code) ? -1 : page_id(code);
   if (rpid >= p.num_pages) rpid = -1;
   if (rpid < 0) return;
-  if (tid == 0) {
-    int n = 0, me = 0;
-    for (int j = 0; j < p.NB; ++j) {
-      const int c = p.table[(int64_t)b * p.NB + j];
-      const int pid = page_is_pad(c) ? -1 : page_id(c);
-      if (pid >= 0 && pid < p.num_pages) {
-        if (j == jp) me = n;
-        vpage[n] = pid; vidx[n] = j; ++n;
-      }
-    }
-    nvalid_s = n;
-    mine_s = me;
-  }
+  list_valid_pages(p.table + (int64_t)b * p.NB, p.NB, p.num_pages, jp, vpage, vidx, nullptr, &nvalid_s, &mine_s);
   const int dpieces = p.D / 8;
   if (dpieces < PIECES) {   // head dims below 128 leave the upper pieces of every LDS row at zero
     for (int i = tid; i < 2 * kRawTileBytes / 4; i += kThreads) ((uint32_t*)smem)[i] = 0u;
@@ -2074,8 +2054,18 @@ __global__ __launch_bounds__(kThreads) void raw_claim_value_kernel(GramArgs p) {
 __device__ __forceinline__ int to_fixed26(float v) { return (int)(v * 67108864.f); }
 __device__ __forceinline__ float from_fixed26(int w) { return (float)w * (1.f / 67108864.f); }
 
+#ifdef ZP_PAGE_STAMP
+__device__ long long zp_chain_stamp_buf[(1 << 16) * 12];
+extern "C" int zp_debug_chain_stamps(long long* dst, int n_groups) {
+  return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(zp_chain_stamp_buf), (size_t)n_groups * 12 * 8);
+}
+#define ZP_CSTAMP(i) do { if (tid == 0) { const long long c_ = clock64(); acc_[i] += c_ - last_; last_ = c_; } } while (0)
+#else
+#define ZP_CSTAMP(i) do { } while (0)
+#endif
+
 template <typename T>
-__global__ __launch_bounds__(512) void raw_chain_kernel(GramArgs p) {
+__global__ __launch_bounds__(512, 4) void raw_chain_kernel(GramArgs p) {
   static_assert(T::bytes == 2, "16-bit caches only");
   typedef typename Mfma16<T>::V frag_t;
   constexpr int kT = 512, kW = 8, KSB = kDmax / 16, CT = 32;     // CT chunks per tile
@@ -2092,6 +2082,11 @@ __global__ __launch_bounds__(512) void raw_chain_kernel(GramArgs p) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, col = lane & 31;
+#ifdef ZP_PAGE_STAMP
+  long long acc_[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  long long last_ = clock64();
+  const long long wall0 = wall_clock64();
+#endif
   const int jp = blockIdx.x % p.NB;
   const int h = (blockIdx.x / p.NB) % p.Hkv;
   const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
@@ -2106,15 +2101,7 @@ __global__ __launch_bounds__(512) void raw_chain_kernel(GramArgs p) {
     for (int s = tid; s < p.BS; s += kT) Elem<T>::st(p.r_out, obase + (int64_t)jp * p.BS + s, -INFINITY);
     return;
   }
-  if (tid == 0) {
-    int n = 0;
-    for (int j = 0; j < p.NB; ++j) {
-      const int c = p.table[(int64_t)b * p.NB + j];
-      const int pid = page_is_pad(c) ? -1 : page_id(c);
-      if (pid >= 0 && pid < p.num_pages) { vidx[n] = j; vord[j] = n; ++n; } else vord[j] = -1;
-    }
-    nvalid_s = n;
-  }
+  list_valid_pages(p.table + (int64_t)b * p.NB, p.NB, p.num_pages, jp, nullptr, vidx, vord, &nvalid_s, nullptr);
   __syncthreads();
   const int cpp = p.BS / kChunk;
   const int nchunks = nvalid_s * cpp;
@@ -2148,6 +2135,7 @@ __global__ __launch_bounds__(512) void raw_chain_kernel(GramArgs p) {
       }
       ssq += lane_xor32(ssq);
     }
+    ZP_CSTAMP(0);   // set-up, key loads issued
     const float rn = live ? p.ws_sum[obase + (int64_t)jp * p.BS + slot] : 0.f;
     const float diag = ssq * rn * rn;                 // S_ii, the entry the reference zeroes
     const int own_chunk = my_ord * cpp + slot / kChunk;
@@ -2158,33 +2146,55 @@ __global__ __launch_bounds__(512) void raw_chain_kernel(GramArgs p) {
     __syncthreads();
     if (tid == 0) nlist_s = 0;
     __syncthreads();
-    for (int t = tid; t < Tn; t += kT) {
-      const int jt = t / p.BS;
-      const int ord = vord[jt];
-      if (ord < 0) continue;
-      const int cc = p.ws_col[obase + t] - (jp * p.BS + key0);   // the row key t claimed from
-      if (cc >= 0 && cc < KEYS && key0 + cc < p.BS) {
-        const int i = atomicAdd(&nlist_s, 1);
-        lst_key[i] = (uint32_t)(ord * cpp + (t - jt * p.BS) / kChunk) << 16 | (uint32_t)cc;
-        lst_val[i] = p.ws_val[obase + t];
+    for (int t0 = tid; t0 < Tn; t0 += 4 * kT) {      // four independent loads in flight per thread
+      int cw[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int t = t0 + u * kT;
+        cw[u] = t < Tn ? p.ws_col[obase + t] : -1;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int t = t0 + u * kT;
+        if (t >= Tn) continue;
+        const int jt = t / p.BS;
+        const int ord = vord[jt];
+        if (ord < 0) continue;
+        const int cc = cw[u] - (jp * p.BS + key0);   // the row key t claimed from
+        if (cc >= 0 && cc < KEYS && key0 + cc < p.BS) {
+          const int i = atomicAdd(&nlist_s, 1);
+          lst_key[i] = (uint32_t)(ord * cpp + (t - jt * p.BS) / kChunk) << 16 | (uint32_t)cc;
+          lst_val[i] = p.ws_val[obase + t];
+        }
       }
     }
     __syncthreads();
     const int nlist = nlist_s;
+    ZP_CSTAMP(1);   // claims gathered
 
-    for (int tile = 0; tile < ntiles; ++tile) {
-      const int c0 = tile * CT;
-      // ---- corrections of this tile, and its three planes
-      for (int i = tid; i < CT * KEYS; i += kT) cl[i] = 0;
-      for (int i = tid; i < CT * (kDmax / 4); i += kT) {
+    // the chunk sums of a tile (CT chunks x kDmax floats, two float4 per thread) are requested one
+    // tile ahead and split into the three planes once the tile before is done with them
+    static_assert(CT * (kDmax / 4) == 2 * kT, "two float4 of a tile's chunk sums per thread");
+    float4 pv[2];
+    auto request_planes = [&](int tile) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int i = tid + u * kT;
         const int m = i / (kDmax / 4), q4 = i - m * (kDmax / 4);
-        const int vc = c0 + m;
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        const int vc = tile * CT + m;
+        pv[u] = make_float4(0.f, 0.f, 0.f, 0.f);
         if (vc < nchunks) {
           const int vp = vc / cpp, c = vc - vp * cpp;
-          v = *(const float4*)(chunk_all + ((int64_t)vidx[vp] * cpp + c) * kDmax + q4 * 4);
+          pv[u] = *(const float4*)(chunk_all + ((int64_t)vidx[vp] * cpp + c) * kDmax + q4 * 4);
         }
-        const float f[4] = {v.x, v.y, v.z, v.w};
+      }
+    };
+    auto store_planes = [&]() {
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int i = tid + u * kT;
+        const int m = i / (kDmax / 4), q4 = i - m * (kDmax / 4);
+        const float f[4] = {pv[u].x, pv[u].y, pv[u].z, pv[u].w};
         uint16_t o[4][3];
 #pragma unroll
         for (int q = 0; q < 4; ++q) Split3<T>::run(f[q], o[q]);
@@ -2196,7 +2206,16 @@ __global__ __launch_bounds__(512) void raw_chain_kernel(GramArgs p) {
           *(uint2*)(planes + (pl * CT + m) * ROWH + q4 * 8) = w;
         }
       }
+    };
+    if (ntiles > 0) { request_planes(0); store_planes(); }
+    if (ntiles > 1) request_planes(1);
+    ZP_CSTAMP(2);   // first planes
+    for (int tile = 0; tile < ntiles; ++tile) {
+      const int c0 = tile * CT;
+      // ---- corrections of this tile (its three planes are in LDS)
+      for (int i = tid; i < CT * KEYS / 4; i += kT) ((int4*)cl)[i] = make_int4(0, 0, 0, 0);
       __syncthreads();
+      ZP_CSTAMP(3);   // corrections cleared
       if (half == 0 && live && own_chunk >= c0 && own_chunk < c0 + CT)
         atomicAdd(&cl[(own_chunk - c0) * KEYS + wave * 32 + col], to_fixed26(diag));
       for (int i = tid; i < nlist; i += kT) {
@@ -2206,6 +2225,7 @@ __global__ __launch_bounds__(512) void raw_chain_kernel(GramArgs p) {
           atomicAdd(&cl[(vc - c0) * KEYS + (int)(w & 0xffffu)], to_fixed26(lst_val[i]));
       }
       __syncthreads();
+      ZP_CSTAMP(4);   // corrections added
       // ---- chunk sums of the tile: A = planes (rows = chunks), B = keys
       {
         f32x16_t acc;
@@ -2225,19 +2245,47 @@ __global__ __launch_bounds__(512) void raw_chain_kernel(GramArgs p) {
         }
       }
       __syncthreads();
+      ZP_CSTAMP(5);   // products
+      // the products are done with this tile's planes: the next tile's go in, the one after is requested
+      if (tile + 1 < ntiles) {
+        store_planes();
+        if (tile + 2 < ntiles) request_planes(tile + 2);
+      }
       // ---- the reference's chain: one cache-dtype partial sum per column page
       if (tid < KEYS) {
-        for (int m = 0; m < CT && c0 + m < nchunks; ++m) {
-          if ((c0 + m) % cpp == 0) { total += part; part = 0.f; }
-          part = Elem<T>::rnd(part + __int_as_float(cl[m * KEYS + tid]));
+        int cm = c0 % cpp;                     // where the tile's first chunk lies inside its page
+        const int mend = min(CT, nchunks - c0);
+        for (int m0 = 0; m0 < mend; m0 += 8) {   // eight chunk sums read ahead of the serial chain
+          float v[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) v[u] = m0 + u < mend ? __int_as_float(cl[(m0 + u) * KEYS + tid]) : 0.f;
+#pragma unroll
+          for (int u = 0; u < 8; ++u) {
+            if (m0 + u < mend) {
+              if (cm == 0) { total += part; part = 0.f; }
+              part = Elem<T>::rnd(part + v[u]);
+              cm = cm + 1 == cpp ? 0 : cm + 1;
+            }
+          }
         }
       }
+      ZP_CSTAMP(6);   // next planes stored, chain of thread 0
       __syncthreads();
+      ZP_CSTAMP(7);   // barrier behind the chain
     }
     if (tid < KEYS && key0 + tid < p.BS)
       Elem<T>::st(p.r_out, obase + (int64_t)jp * p.BS + key0 + tid, total + part);
   }
+#ifdef ZP_PAGE_STAMP
+  if (tid == 0 && blockIdx.x < (1 << 16)) {
+    long long* dst = zp_chain_stamp_buf + (int64_t)blockIdx.x * 12;
+    for (int i = 0; i < 8; ++i) dst[i] = acc_[i];
+    dst[10] = wall0;
+    dst[11] = wall_clock64() - wall0;
+  }
+#endif
 }
+#undef ZP_CSTAMP
 
 // ------------------------------------------------------------------ softmax epilogue
 // One workgroup per (layer, sequence, head) row of T logits:
