@@ -59,12 +59,14 @@ int zp_store_query(const void* query, void* query_cache, const int32_t* slot_map
  * k_cache (L, num_pages, BS, Hkv, D), query_cache (L, max_seqs, W, Hq, D), both
  * contiguous in their last two axes; scores_out (L, B, Hkv, NB, BS) contiguous, in the
  * cache dtype; logits_out NULL or (L, B, Hq, W, NB, BS) contiguous.
- * workspace: zp_attention_score_workspace() bytes of device scratch -- an upper bound over
- * the dtypes.  With 16-bit caches, no logits_out, a positive scale and at most 2560 tokens per
- * sequence that scratch lets the library keep the rounded logits in registers and sweep K once
- * (fp32 window partials per block of 32 query rows go through the scratch); with less scratch
- * (NULL is fine up to 128 window x group rows) the same entry point sweeps K three times.  The
- * two kernels round at the same points and differ only in the fp32 order of the row sums. */
+ * workspace: zp_attention_score_workspace_for(..., dtype) bytes of device scratch
+ * (zp_attention_score_workspace(): the upper bound over the dtypes).  With no logits_out, a
+ * positive scale and at most 2560 tokens per sequence that scratch lets the library keep the
+ * logits in registers and sweep K once (fp32 window partials per block of 32 query rows -- 16
+ * for fp32 caches -- go through the scratch); with less scratch (NULL is fine up to 128 window x
+ * group rows) the same entry point sweeps K three times (twice for fp32 caches).  The kernels
+ * round at the same points and differ only in the fp32 order of the row sums (fp32 caches: also
+ * in the last bit of the probabilities, e / sum against 2^(x log2 e - log2 sum)). */
 int zp_attention_score(const void* k_cache, const void* query_cache, const int32_t* seq_idx,
                        const int32_t* block_table, void* scores_out, void* logits_out,
                        int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
@@ -75,6 +77,8 @@ int zp_attention_score(const void* k_cache, const void* query_cache, const int32
                        int64_t workspace_bytes, void* stream);
 int64_t zp_attention_score_workspace(int32_t L, int32_t B, int32_t NB, int32_t BS,
                                      int32_t Hkv, int32_t Hq, int32_t W);
+int64_t zp_attention_score_workspace_for(int32_t L, int32_t B, int32_t NB, int32_t BS,
+                                         int32_t Hkv, int32_t Hq, int32_t W, int32_t dtype);
 
 /* global_score(reduced_scores, score_cache, block_table, compressed, decay_factor,
  *              activate_method)

@@ -364,6 +364,43 @@ def test_attention_score_one_sweep_matches_three_sweeps(dev, dtype, shape, reduc
     assert (one.cpu()[pad] == 0).all()     # pad pages score exactly 0
 
 
+@pytest.mark.parametrize("shape", [
+    dict(Hkv=8, Hq=16, W=32, nb_choices=(9, 10)),           # group 2 (configs[2]): four blocks of 16 rows, 36-40 tiles
+    dict(Hkv=2, Hq=8, W=16, nb_choices=(2, 5, 9)),          # group 4
+    dict(Hkv=1, Hq=7, W=24, nb_choices=(3, 4)),             # group 7 padded to 8: a window spans two lane groups
+    dict(Hkv=1, Hq=16, W=5, nb_choices=(2, 3)),             # group 16: a block is one window
+    dict(Hkv=3, Hq=3, W=8, nb_choices=(1, 2)),              # no group, half a block of rows
+    dict(Hkv=2, Hq=4, W=32, D=64, BS=128, nb_choices=(7, 20)),   # two tiles per page, 64-wide heads
+    dict(Hkv=2, Hq=8, W=32, BS=192, nb_choices=(2, 6)),     # three tiles per page
+    dict(Hkv=2, Hq=4, W=12, D=32, BS=64, nb_choices=(5, 33)),    # one tile per page, 32-wide heads
+])
+@pytest.mark.parametrize("reduced", ["mean", "max"])
+def test_attention_score_fp32_one_sweep_matches_two_sweeps(dev, shape, reduced):
+    """fp32 caches, sequences of at most 2560 tokens: the kernel that keeps the logits in registers
+    (one sweep over K, blocks of 16 query rows) against the kernel that recomputes them and against
+    the oracle, to the fp32 tolerance."""
+    from zipage_amd import _lib
+    from zipage_amd.kernel import attention_score
+    shape = dict(shape)
+    nb = shape.pop("nb_choices")
+    s = _setup(79, torch.float32, L=2, B=4, nb_choices=nb, num_pages=140, **shape)
+    args = tuple(a.to(dev) for a in (s["k"], s["q"], s["seq_idx"], s["enc"]))
+    L, _, BS, Hkv, _ = s["k"].shape
+    B, NB = s["enc"].shape
+    Hq, W = s["q"].shape[3], s["q"].shape[2]
+    lib = _lib.load()
+    need = lib.zp_attention_score_workspace_for(L, B, NB, BS, Hkv, Hq, W, 2)
+    assert need == L * B * Hkv * -(-W * max(1, 1 << (Hq // Hkv - 1).bit_length()) // 16) * NB * BS * 4
+    assert need <= lib.zp_attention_score_workspace(L, B, NB, BS, Hkv, Hq, W)
+    one = attention_score(*args, reduced=reduced)
+    two = _score_three_sweeps(*args, reduced=reduced)
+    _rel_close(one, two.cpu(), rel=1e-4, abs_floor=1e-9)
+    want = O.attention_score(s["k"], s["q"], s["seq_idx"], s["enc"], reduced=reduced)
+    _rel_close(one, want, rel=1e-3, abs_floor=1e-9)
+    pad = (s["enc"] == -1).view(1, -1, 1, s["enc"].shape[1], 1).expand_as(want)
+    assert (one.cpu()[pad] == 0).all()     # pad pages score exactly 0
+
+
 def test_attention_score_long_rows_take_three_sweeps(dev):
     """More than 2560 tokens do not fit the registers: same entry point, three sweeps."""
     from zipage_amd.kernel import attention_score

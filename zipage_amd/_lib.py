@@ -79,6 +79,7 @@ I64_RETURNING = {
     "zp_compress_layers_workspace": [i32, i32, i32, i32, i32, i32, i32, i32,
                                      C.POINTER(CompressConfigC), i32],
     "zp_attention_score_workspace": [i32, i32, i32, i32, i32, i32, i32],
+    "zp_attention_score_workspace_for": [i32, i32, i32, i32, i32, i32, i32, i32],
     "zp_redundancy_raw_workspace": [i32, i32, i32, i32, i32],
 }
 EXPORTS = sorted(list(SIGNATURES) + list(I64_RETURNING) + ["zp_abi_version", "zp_last_error"])

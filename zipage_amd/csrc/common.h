@@ -32,6 +32,8 @@ void zp_set_error(const char* fmt, ...);
 
 // Scratch zp_attention_score cannot do without (it takes the three-sweep kernel when the caller
 // brings less than zp_attention_score_workspace() asks for).  Library-internal.
+extern "C" int64_t zp_attention_score_workspace_for(int32_t L, int32_t B, int32_t NB, int32_t BS,
+                                                    int32_t Hkv, int32_t Hq, int32_t W, int32_t dtype);
 int64_t zp_attention_score_workspace_floor(int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
                                            int32_t Hq, int32_t W);
 

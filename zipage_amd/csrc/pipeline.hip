@@ -44,9 +44,8 @@ Plan make_plan(int L, int B, int NB, int BS, int Hkv, int Hq, int W, int dtype,
                   ? take(n * es) : -1;
   p.red = c->use_redundancy ? take(n * es) : -1;
   p.flag = own_flag ? take(n) : -1;
-  p.score_ws_bytes = (lean || dtype == ZP_F32)
-                         ? zp_attention_score_workspace_floor(L, B, NB, BS, Hkv, Hq, W)
-                         : zp_attention_score_workspace(L, B, NB, BS, Hkv, Hq, W);
+  p.score_ws_bytes = lean ? zp_attention_score_workspace_floor(L, B, NB, BS, Hkv, Hq, W)
+                          : zp_attention_score_workspace_for(L, B, NB, BS, Hkv, Hq, W, dtype);
   p.score_ws = p.score_ws_bytes ? take(p.score_ws_bytes) : -1;
   p.raw_ws_bytes = (c->use_redundancy && !c->lightning) ? zp_redundancy_raw_workspace(L, B, NB, BS, Hkv) : 0;
   p.raw_ws = p.raw_ws_bytes ? take(p.raw_ws_bytes) : -1;

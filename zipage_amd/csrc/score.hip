@@ -1112,6 +1112,279 @@ __global__ __launch_bounds__(kThreads, 2) void score_resident_kernel(ScoreArgs p
 #undef ZP_STAMP
 }
 
+// ------------------------------------------------------------------ fp32 caches: one sweep
+// The same structure for fp32 caches.  An fp32 logit fills a register, so a unit is 16 query rows
+// (v_mfma_f32_16x16x4_f32: lane (c, q) = (lane % 16, lane / 16) holds row / token c of the
+// operands at contraction index q and rows 4 q .. 4 q + 3 of token c of the result); wave t owns
+// tokens [64 i + 16 t, +16) of every 64-token tile i, four logits per tile and lane, 160 registers
+// for 40 tiles.  fp32 has no rounding chain: exp(logit - max) replaces the logit in its register
+// while the row sums accumulate, and the output pass is one multiplication per entry.
+//   * The contraction index is free as long as both operands agree: step 4 j + i of lane group q
+//     takes element 16 j + 4 q + i, so a lane's operands for four steps are 16 consecutive bytes.
+//   * A load instruction fills 1 KB of LDS with two key rows (32 pieces of 16 bytes each): piece g
+//     of row r of a pair at ((g / 16) * 32 + (g % 16) * 2 + r) * 16, pairs 1056 bytes apart, so the
+//     sixteen lanes that read one piece of sixteen consecutive rows fall into sixteen different
+//     16-byte bank groups.
+constexpr int kF32Tiles = 40;              // 64-token tiles of a row: at most 2 560 tokens
+constexpr int kF32Pair = 1056;             // bytes from one pair of staged key rows to the next
+constexpr int kF32Sub = 8 * kF32Pair;      // a wave's block of 16 key rows
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+template <int GPC, int RMAXC, int TPP>
+__global__ __launch_bounds__(kThreads, 2) void score_resident_f32_kernel(ScoreArgs p) {
+  const int GpV = GPC > 0 ? GPC : p.Gp;
+  const int gsV = GPC == 8 ? 3 : GPC == 4 ? 2 : GPC == 2 ? 1 : p.gs;
+  const bool rmaxV = RMAXC >= 0 ? (RMAXC != 0) : (p.reduce_max != 0);
+
+  extern __shared__ __align__(16) char smem[];
+  float* stat = (float*)(smem + kWaves * 2 * kF32Sub);   // [kWaves][16] row maxima, then row sums
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kq = lane >> 4, col = lane & 15;
+  // unit -> (item, row block), as in the 16-bit kernel: the row blocks of an item side by side on
+  // one XCD
+  const int xcd = blockIdx.x & 7, loc = blockIdx.x >> 3;
+  const int rb = loc % p.RB;
+  const int item = (loc / p.RB) * 8 + xcd;
+  if (item >= p.n_items) return;
+  const int h = item % p.Hkv;
+  const int b = (item / p.Hkv) % p.B;
+  const int l = item / (p.Hkv * p.B);
+  const int Tn = p.NB * p.BS;
+
+  // per-wave list of usable pages: entry n in lane n as (page id, table index | last << 30)
+  const int code = lane < p.NB ? p.table[(int64_t)b * p.NB + lane] : -1;
+  int seq = p.seq_idx[b];
+  int2 myinfo;
+  int nvalid;
+  {
+    const int pid = page_is_pad(code) ? -1 : page_id(code);
+    const bool ok = pid >= 0 && pid < p.num_pages;
+    const unsigned long long okm = __builtin_amdgcn_ballot_w64(ok);
+    nvalid = __builtin_popcountll(okm);
+    const int dst = ok ? __builtin_popcountll(okm & lanemask_lt())
+                       : nvalid + __builtin_popcountll(~okm & lanemask_lt());
+    myinfo.x = __builtin_amdgcn_ds_permute(dst << 2, pid);
+    myinfo.y = __builtin_amdgcn_ds_permute(dst << 2, lane | (page_is_last(code) ? (1 << 30) : 0));
+  }
+  const int dpieces = p.D / 4;               // 16-byte pieces of a key row
+  char* kb = smem + wave * 2 * kF32Sub;      // this wave's two key blocks
+  if (dpieces < 32) {   // the tail of every staged row must read as zero
+    for (int i = lane; i < 2 * kF32Sub / 4; i += 64) ((uint32_t*)kb)[i] = 0u;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  }
+  const bool seq_ok = seq >= 0 && seq < p.max_seqs;
+  if (!seq_ok) seq = 0;
+
+  const int tiles_per_page = TPP > 0 ? TPP : p.BS / 64;
+  const int ntiles = nvalid * tiles_per_page;
+  auto tile_page = [&](int tile) { return tile / (TPP > 0 ? TPP : tiles_per_page); };
+  auto page_word = [&](int v, int vp) {   // entry vp of the list, wave-uniform
+    if constexpr (TPP > 0) return __builtin_amdgcn_readlane(v, vp);
+    else return __builtin_amdgcn_readfirstlane(__builtin_amdgcn_ds_bpermute(vp << 2, v));
+  };
+  const int64_t k_row = (int64_t)p.Hkv * p.D * 4;
+  const char* kbase = p.k + (l * p.k_sl) * 4 + (int64_t)h * p.D * 4;
+  const int wtok = wave * 16;   // this wave's tokens inside a tile
+
+  // ---- staging: a load instruction moves two rows; lane -> (row of the pair, piece)
+  const int st_g = (lane >> 5) * 16 + ((lane & 31) >> 1), st_r = lane & 1;
+  const int st_off = (int)(st_r * k_row + st_g * 16);
+  const bool st_ok = st_g < dpieces;
+  const int pair_step = (int)(2 * k_row);
+  typedef void __attribute__((address_space(3))) * lptr_t;
+  auto issue = [&](int tile, char* buf) {
+    const int vp = tile_page(tile);
+    const int pid = page_word(myinfo.x, vp);
+    const int toff = (tile - vp * tiles_per_page) * 64 + wtok;
+    const char* src = kbase + (int64_t)pid * p.k_sp * 4 + (int64_t)toff * k_row;
+    const __amdgpu_buffer_rsrc_t rs =
+        __builtin_amdgcn_make_buffer_rsrc((void*)src, 0, (int)(16 * k_row), 0x00020000);
+    if (st_ok) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lptr_t)(buf + i * kF32Pair), 16, st_off,
+                                                 i * pair_step, 0, 0);
+    }
+  };
+  // operands of steps 4 j .. 4 j + 3 of this lane's token: base + (j / 4) * 512 + (j % 4) * 128
+  const int rd_off = (col >> 1) * kF32Pair + kq * 32 + (col & 1) * 16;
+
+  if (ntiles > 0) issue(0, kb);
+  if (ntiles > 1) issue(1, kb + kF32Sub);
+
+  // ---- A operands: query row `col` of this block at this lane group's contraction indices
+  f32x4_t aq[8];
+  {
+    const int mrow = rb * 16 + col;
+    const int a_w = mrow >> gsV, a_g = mrow & (GpV - 1);
+    const bool a_ok = seq_ok && a_w < p.W && a_g < p.G;
+    const char* qrow = p.q + ((int64_t)l * p.q_sl + (int64_t)seq * p.q_ss +
+                              ((int64_t)a_w * p.Hq + (int64_t)h * p.G + a_g) * p.D) * 4;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k0 = 16 * j + 4 * kq;
+      if (a_ok && k0 < p.D) aq[j] = *(const f32x4_t*)(qrow + (int64_t)k0 * 4);
+      else aq[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+  // the sweep counts its own loads with s_waitcnt: the query loads must be out of the way.  They
+  // were issued after the first two key blocks, so waiting for them waits for those blocks too.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int j = 0; j < 8; ++j) asm volatile("" : "+v"(aq[j]));
+
+  const int row0 = rb * 16 + kq * 4;   // rows of this lane: row0 + r
+  float lg[kF32Tiles * 4];
+  float run[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) run[r] = -INFINITY;
+
+  // ---- the sweep: products, causal mask, running maximum, logits into registers; the products
+  // of block it+1 are issued before the vector work on block it
+  auto products = [&](int it) {
+    const char* cur = kb + (it & 1) * kF32Sub + rd_off;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j0 = 0; j0 < 8; j0 += 4) {
+      f32x4_t bf[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bf[j] = *(const f32x4_t*)(cur + ((j0 + j) >> 2) * 512 + ((j0 + j) & 3) * 128);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(aq[j0 + j][i], bf[j][i], acc, 0, 0, 0);
+      }
+    }
+    return acc;
+  };
+  f32x4_t acc_cur = {0.f, 0.f, 0.f, 0.f};
+  if (ntiles > 0) acc_cur = products(0);
+  // every operand of block 0 is in registers: block 2 may overwrite it
+  asm volatile("" ::: "memory");
+  if (ntiles > 2) issue(2, kb);
+#pragma unroll
+  for (int it = 0; it < kF32Tiles; ++it) {
+    if (it < ntiles) {
+      f32x4_t acc_next = {0.f, 0.f, 0.f, 0.f};
+      if (it + 1 < ntiles) {
+        // block it+1 has landed once at most the 8 loads of block it+2 are outstanding
+        if (it + 1 >= 2) {
+          if (it + 2 < ntiles) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+          else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        acc_next = products(it + 1);
+        asm volatile("" ::: "memory");
+        if (it + 3 < ntiles) issue(it + 3, kb + ((it + 1) & 1) * kF32Sub);
+      }
+      f32x4_t acc = acc_cur;
+      const int vp = tile_page(it);
+      const int vs = page_word(myinfo.y, vp);
+      const int toff = (it - vp * tiles_per_page) * 64 + wtok;
+      if (((vs >> 30) & 1) && (toff + 15 > p.BS - p.W)) {   // causal mask: tail of the last page
+        const int slot = toff + col;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int w = (row0 + r) >> gsV;
+          if (slot > p.BS - p.W + w) acc[r] = -INFINITY;
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        run[r] = vmax(run[r], acc[r]);
+        lg[it * 4 + r] = acc[r] * p.scale;
+      }
+      if (it + 1 < ntiles) acc_cur = acc_next;
+    }
+  }
+
+  // ---- row maximum over the 16 tokens of a lane group and the four waves
+  float mx[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float v = row16_max(run[r]);
+    run[r] = v;
+    if (col == 0) stat[wave * 16 + kq * 4 + r] = v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float v = run[r];
+#pragma unroll
+    for (int w2 = 1; w2 < kWaves; ++w2) v = fmaxf(v, stat[((wave + w2) % kWaves) * 16 + kq * 4 + r]);
+    mx[r] = v * p.scale;
+  }
+  __syncthreads();
+
+  // ---- exp(logit - max) back into the registers, row sums
+#pragma unroll
+  for (int r = 0; r < 4; ++r) run[r] = 0.f;
+#pragma unroll
+  for (int it = 0; it < kF32Tiles; ++it) {
+    if (it < ntiles) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float e = exp_neg(lg[it * 4 + r] - mx[r]);
+        lg[it * 4 + r] = e;
+        run[r] += e;
+      }
+    }
+  }
+  float inv[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float v = row16_sum(run[r]);
+    if (col == 0) stat[wave * 16 + kq * 4 + r] = v;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    // the four waves' sums are added in wave order, whichever wave does it
+    float v = stat[kq * 4 + r];
+#pragma unroll
+    for (int w2 = 1; w2 < kWaves; ++w2) v += stat[w2 * 16 + kq * 4 + r];
+    const int m = row0 + r;
+    const bool ok = (m >> gsV) < p.W && (m & (GpV - 1)) < p.G;
+    inv[r] = ok ? 1.f / v : 0.f;   // rows outside the window or group contribute 0 (probabilities are >= 0)
+  }
+
+  // ---- output: p = e / sum, group maximum, this block's share of the window sum (or maximum)
+  float* part = p.part + ((int64_t)item * p.RB + rb) * Tn + wtok + col;
+#pragma unroll
+  for (int it = 0; it < kF32Tiles; ++it) {
+    if (it < ntiles) {
+      float pv[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) pv[r] = lg[it * 4 + r] * inv[r];
+      // a lane's four rows are consecutive: groups of 1, 2 or 4 rows are whole inside the lane,
+      // groups of 8 / 16 rows span two / four lane groups
+      float red;
+      if (GpV == 1) {
+        red = rmaxV ? vmax(vmax(pv[0], pv[1]), vmax(pv[2], pv[3])) : (pv[0] + pv[1]) + (pv[2] + pv[3]);
+      } else if (GpV == 2) {
+        const float g0 = vmax(pv[0], pv[1]), g1 = vmax(pv[2], pv[3]);
+        red = rmaxV ? vmax(g0, g1) : g0 + g1;
+      } else {
+        red = vmax(vmax(pv[0], pv[1]), vmax(pv[2], pv[3]));
+      }
+      {
+        const float o = lane_xor16(red);
+        red = (GpV >= 8 || rmaxV) ? vmax(red, o) : red + o;
+      }
+      {
+        const float o = lane_xor32(red);
+        red = (GpV >= 16 || rmaxV) ? vmax(red, o) : red + o;
+      }
+      const int vp = tile_page(it);
+      const int j = page_word(myinfo.y, vp) & 0xffff;
+      const int toff = (it - vp * tiles_per_page) * 64;
+      if (kq == 0) __builtin_nontemporal_store(red, part + j * p.BS + toff);
+    }
+  }
+}
+
 // Adds the row blocks' window partials of every (layer, sequence, head) in block order, divides by
 // the window length, rounds to the cache dtype; pad pages score exactly 0.
 template <typename T>
@@ -1185,15 +1458,41 @@ static int64_t sweep_workspace(int L, int B, int NB, int BS, int Hkv, int Hq, in
   return (int64_t)L * B * Hkv * NB * BS * 4;
 }
 
+// fp32 caches: pages in whole 64-token tiles, at most 40 tiles, groups of at most 16 rows.
+static bool resident_f32_shape_ok(int NB, int BS, int Hkv, int Hq, int D) {
+  if (Hkv <= 0 || Hq <= 0 || Hq % Hkv != 0) return false;
+  const int Gp = pow2_ceil(Hq / Hkv);
+  return BS % 64 == 0 && (int64_t)NB * (BS / 64) <= kF32Tiles && NB <= 64 && Gp <= 16 &&
+         D <= kDmax && D % 4 == 0;
+}
+
+// Bytes of fp32 window partials the one-sweep kernel of a dtype needs (0: the shape takes three
+// sweeps): one partial per token and block of 32 (16-bit caches) or 16 (fp32) query rows.
+static int64_t resident_need(int L, int B, int NB, int BS, int Hkv, int Hq, int W, int dtype) {
+  if (Hkv <= 0 || Hq <= 0 || Hq % Hkv != 0) return 0;
+  const int Gp = pow2_ceil(Hq / Hkv);
+  if (dtype == ZP_F32) {
+    if (!resident_f32_shape_ok(NB, BS, Hkv, Hq, kDmax)) return 0;
+    return (int64_t)L * B * Hkv * ((W * Gp + 15) / 16) * NB * BS * 4;
+  }
+  if (!resident_shape_ok(NB, BS, Hkv, Hq, kDmax)) return 0;
+  return (int64_t)L * B * Hkv * ((W * Gp + 31) / 32) * NB * BS * 4;
+}
+
+extern "C" int64_t zp_attention_score_workspace_for(int32_t L, int32_t B, int32_t NB, int32_t BS,
+                                                    int32_t Hkv, int32_t Hq, int32_t W, int32_t dtype) {
+  if (Hkv <= 0 || Hq <= 0 || L < 0 || B < 0 || NB <= 0 || BS <= 0 || W <= 0) return 0;
+  if (dtype < ZP_BF16 || dtype > ZP_F32) return -1;
+  const int64_t floor_bytes = sweep_workspace(L, B, NB, BS, Hkv, Hq, W);
+  const int64_t res = resident_need(L, B, NB, BS, Hkv, Hq, W, dtype);
+  return res > floor_bytes ? res : floor_bytes;
+}
+
 extern "C" int64_t zp_attention_score_workspace(int32_t L, int32_t B, int32_t NB, int32_t BS,
                                                 int32_t Hkv, int32_t Hq, int32_t W) {
-  if (Hkv <= 0 || Hq <= 0 || L < 0 || B < 0 || NB <= 0 || BS <= 0 || W <= 0) return 0;
-  const int64_t floor_bytes = sweep_workspace(L, B, NB, BS, Hkv, Hq, W);
-  if (!resident_shape_ok(NB, BS, Hkv, Hq, kDmax)) return floor_bytes;
-  const int Gp = pow2_ceil(Hq / Hkv);
-  const int64_t RB = (W * Gp + 31) / 32;
-  const int64_t res = (int64_t)L * B * Hkv * RB * NB * BS * 4;   // fp32 window partials per row block
-  return res > floor_bytes ? res : floor_bytes;
+  const int64_t a = zp_attention_score_workspace_for(L, B, NB, BS, Hkv, Hq, W, ZP_BF16);
+  const int64_t b = zp_attention_score_workspace_for(L, B, NB, BS, Hkv, Hq, W, ZP_F32);
+  return a > b ? a : b;
 }
 
 int64_t zp_attention_score_workspace_floor(int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
@@ -1245,12 +1544,13 @@ extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
   const int64_t need = sweep_workspace(L, B, NB, BS, Hkv, Hq, W);
   // One sweep over K with the logits in registers when the shape allows it and the caller
   // brought the scratch for the window partials; three sweeps otherwise.
-  const int64_t res_need = (int64_t)L * B * Hkv * RB * NB * BS * 4;
-  const bool resident = es == 2 && !logits_out && softmax_scale > 0.f &&
-                        resident_shape_ok(NB, BS, Hkv, Hq, D) && workspace &&
-                        workspace_bytes >= res_need && ((uintptr_t)workspace % 4) == 0 &&
-                        (int64_t)L * B * Hkv < ((int64_t)1 << 28);
-  ZP_REQUIRE(resident || need == 0 || (workspace && workspace_bytes >= need),
+  const int64_t res_need = resident_need(L, B, NB, BS, Hkv, Hq, W, dtype);
+  const bool res_common = !logits_out && softmax_scale > 0.f && workspace && res_need > 0 &&
+                          workspace_bytes >= res_need && ((uintptr_t)workspace % 16) == 0 &&
+                          (int64_t)L * B * Hkv < ((int64_t)1 << 27);
+  const bool resident = es == 2 && res_common && resident_shape_ok(NB, BS, Hkv, Hq, D);
+  const bool resident32 = es == 4 && res_common && resident_f32_shape_ok(NB, BS, Hkv, Hq, D);
+  ZP_REQUIRE(resident || resident32 || need == 0 || (workspace && workspace_bytes >= need),
              "attention_score: workspace of %lld bytes required", (long long)need);
 
   ScoreArgs a;
@@ -1288,6 +1588,25 @@ extern "C" int zp_attention_score(const void* k_cache, const void* query_cache,
     if (dtype == ZP_BF16) ZP_RESIDENT_LAUNCH(BF16);
     else ZP_RESIDENT_LAUNCH(F16);
 #undef ZP_RESIDENT_LAUNCH
+    ZP_LAUNCH_CHECK();
+    return ZP_OK;
+  }
+  if (resident32) {
+    a.RB = (W * Gp + 15) / 16;
+    const size_t smem = (size_t)kWaves * 2 * kF32Sub + sizeof(float) * kWaves * 16;
+    const unsigned units = (unsigned)(((int64_t)a.n_items + 7) / 8 * 8 * a.RB);
+    const dim3 cgrid((unsigned)a.n_items, (unsigned)((NB * BS / 4 + 255) / 256));
+    void (*fn)(ScoreArgs) = score_resident_f32_kernel<0, -1, 0>;
+    if (Gp == 2 && !a.reduce_max && BS == 256) fn = score_resident_f32_kernel<2, 0, 4>;
+    else if (Gp == 4 && !a.reduce_max && BS == 256) fn = score_resident_f32_kernel<4, 0, 4>;
+    if (hipFuncSetAttribute((const void*)fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) !=
+        hipSuccess) {
+      zp_set_error("attention_score: cannot reserve %zu bytes of LDS", smem);
+      return ZP_EHIP;
+    }
+    hipLaunchKernelGGL(fn, dim3(units), dim3(kThreads), smem, st, a);
+    hipLaunchKernelGGL(score_combine_kernel<F32>, cgrid, dim3(256), 0, st, a.part, scores_out, block_table,
+                       B, NB, BS, Hkv, a.RB, W, num_pages, a.reduce_max);
     ZP_LAUNCH_CHECK();
     return ZP_OK;
   }

@@ -41,7 +41,7 @@ def attention_score(k_cache: torch.Tensor, query_cache: torch.Tensor, seq_idx: t
     if L == 0 or B == 0:  # nothing to score: empty outputs, as the torch ops would give
         return (scores, logits) if return_logits else scores
     lib = _lib.load()
-    ws_bytes = lib.zp_attention_score_workspace(L, B, NB, BS, Hkv, Hq, W)
+    ws_bytes = lib.zp_attention_score_workspace_for(L, B, NB, BS, Hkv, Hq, W, _lib.dtype_tag(k_cache))
     ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8) if ws_bytes else None
     _lib.call("zp_attention_score", _lib.dev_ptr(k_cache), _lib.dev_ptr(query_cache),
               _lib.dev_ptr(seq_idx), _lib.dev_ptr(block_table), _lib.dev_ptr(scores),
