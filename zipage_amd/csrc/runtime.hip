@@ -14,4 +14,4 @@ void zp_set_error(const char* fmt, ...) {
 
 extern "C" const char* zp_last_error(void) { return g_err; }
 
-extern "C" int zp_abi_version(void) { return 3; }
+extern "C" int zp_abi_version(void) { return 4; }

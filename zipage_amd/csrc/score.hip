@@ -5,12 +5,14 @@
 // to the cache dtype), so bf16/fp16 results agree with it to the last bit except where fp32
 // accumulation order moves a value across a rounding boundary.
 //
-// Two kernels:
+// Three kernels:
 //   score_resident_kernel  16-bit caches, at most 2560 tokens per sequence, no logits requested:
 //       ONE sweep over K.  A workgroup is one block of 32 query rows of a (layer, sequence, head);
 //       its rounded logits stay in registers (two per word) and the row maximum, the row sum and
 //       the output come from the registers.  Described above the kernel.
-//   score_kernel           everything else (fp32 caches, longer sequences, logits, no scratch):
+//   score_resident_f32_kernel  the same for fp32 caches: blocks of 16 query rows, one fp32 logit
+//       per register, v_mfma_f32_16x16x4_f32.  Described above the kernel.
+//   score_kernel           everything else (longer sequences, logits, no scratch):
 //       one workgroup per (layer, sequence, kv head).  The softmax normaliser spans the whole
 //       sequence, so it makes three passes over the sequence's pages, recomputing QK^T each time:
 //         pass 1  row maximum of the (rounded) logits,
@@ -21,7 +23,7 @@
 //       fp32 caches take passes 1 and 2 in one sweep.  K tiles are staged through double-buffered
 //       LDS; passes 2 and 3 re-read K from L2 / Infinity Cache.
 //
-// MFMA tiling (wave64, 32x32 tiles), both kernels: the A operand is a block of 32 query rows, row
+// MFMA tiling (wave64, 32x32 tiles), score_kernel and score_resident_kernel: the A operand is a block of 32 query rows, row
 // m = w*Gp + g (Gp = GQA group padded to a power of two), held in registers; the B operand is 32
 // tokens of K read from LDS.  In the 32x32 accumulator layout a lane owns one token column and
 // 16 rows ((r/4)*8 + (lane/32)*4 + r%4), so with this row order the group maximum is taken inside
