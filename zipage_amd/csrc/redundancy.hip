@@ -594,37 +594,62 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
   unsigned long long* l_claim = l_corr + kPage32Rows;       // (claimed index + 1) << 32 | value bits
   float* l_sum = (float*)(l_claim + kPage32Rows);
   float* l_csum = l_sum + kPage32Rows;                        // [4][256] column sums per distance
+  int* l_code = (int*)(l_csum + 4 * kPage32Rows);             // [NB] the block table row
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int half = lane >> 5, col = lane & 31;
-  const int jp = blockIdx.x % p.NB;
-  const int h = (blockIdx.x / p.NB) % p.Hkv;
-  const int b = (blockIdx.x / (p.NB * p.Hkv)) % p.B;
-  const int l = blockIdx.x / (p.NB * p.Hkv * p.B);
+  const int tid0 = threadIdx.x;
+  // a workgroup walks the pages of one (layer, sequence, kv head) row: the next page's keys are
+  // requested into registers under the tiles of this one (a page fills the LDS a CU has, so
+  // nothing else could overlap its load)
+  const int h = blockIdx.x % p.Hkv;
+  const int b = (blockIdx.x / p.Hkv) % p.B;
+  const int l = blockIdx.x / (p.Hkv * p.B);
   const int Tn = p.NB * p.BS;
-  const int64_t obase = (((int64_t)l * p.B + b) * p.Hkv + h) * Tn + (int64_t)jp * p.BS;
-
-  const int code = p.table[(int64_t)b * p.NB + jp];
-  int rpid = page_is_pad(code) ? -1 : page_id(code);
-  if (rpid >= p.num_pages) rpid = -1;
-  if (rpid < 0) {
-    for (int s = tid; s < p.BS; s += kPage32Threads) Elem<T>::st(p.r_out, obase + s, -INFINITY);
-    return;
-  }
+  const int64_t rowbase = (((int64_t)l * p.B + b) * p.Hkv + h) * Tn;
   const int dpieces = p.D / 4;
   const int64_t k_row = (int64_t)p.Hkv * p.D * 4;
-  const char* page = p.k + (l * p.k_sl + (int64_t)rpid * p.k_sp) * 4 + (int64_t)h * p.D * 4;
+  const char* layer = p.k + l * p.k_sl * 4 + (int64_t)h * p.D * 4;
 
-  // ---- stage: all loads of the page in flight, then norms and the normalised copy
-  {
-    const int piece = tid % PIECES, row0 = tid / PIECES;
-    float4 raw[ITERS];
+  for (int j = tid0; j < p.NB; j += kPage32Threads) l_code[j] = p.table[(int64_t)b * p.NB + j];
+  __syncthreads();
+  auto page_of = [&](int j) {     // page id of table entry j, or -1 (uniform)
+    const int code = __builtin_amdgcn_readfirstlane(l_code[j]);
+    const int pid = page_is_pad(code) ? -1 : page_id(code);
+    return pid < p.num_pages ? pid : -1;
+  };
+  auto next_valid = [&](int j) {
+    while (j < p.NB && page_of(j) < 0) ++j;
+    return j;
+  };
+  for (int j = 0; j < p.NB; ++j) {      // entries without a page score -inf
+    if (page_of(j) >= 0) continue;
+    for (int s = tid0; s < p.BS; s += kPage32Threads) Elem<T>::st(p.r_out, rowbase + (int64_t)j * p.BS + s, -INFINITY);
+  }
+  float4 raw[ITERS];
+  auto request = [&](int j, int piece, int prow0) {
+    const char* page = layer + (int64_t)page_of(j) * p.k_sp * 4;
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
-      const int row = it * ROWS_PER_IT + row0;
+      const int row = it * ROWS_PER_IT + prow0;
       raw[it] = *(const float4*)(page + (int64_t)(row < p.BS ? row : 0) * k_row +
                                  (piece < dpieces ? piece : 0) * 16);
     }
+  };
+  int jp = next_valid(0);
+  if (jp < p.NB) request(jp, tid0 % PIECES, tid0 / PIECES);
+#pragma unroll 1
+  while (jp < p.NB) {
+  // The thread id is made opaque once per page: what is derived from it (LDS addresses, row
+  // indices) is then computed where a page uses it, not before the loop and held in registers
+  // through all of it, where the prefetched page needs them.
+  int tid = tid0;
+  asm volatile("" : "+v"(tid));
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = lane >> 5, col = lane & 31;
+  const int piece = tid % PIECES, prow0 = tid / PIECES;
+  const int64_t obase = rowbase + (int64_t)jp * p.BS;
+  // ---- stage: norms and the normalised copy of the page requested a page ago
+  {
+    const int row0 = prow0;
     if (tid < kPage32Rows) { l_corr[tid] = 0ull; l_claim[tid] = 0ull; }
 #pragma unroll
     for (int it = 0; it < ITERS; ++it) {
@@ -638,6 +663,8 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
     }
   }
   __syncthreads();
+  const int nj = next_valid(jp + 1);
+  if (nj < p.NB) request(nj, piece, prow0);
 
   // ---- Gram tiles, every unordered pair of 32-key blocks once: wave a multiplies its block with
   // the blocks (a + d) mod n, d = 0 .. n/2 (the last distance only for the lower half of the
@@ -736,6 +763,9 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
       if (ran) sv += l_csum[(d - 1) * kPage32Rows + i];
     }
     Elem<T>::st(p.r_out, obase + i, sv - from_fixed32(l_corr[i]));
+  }
+  __syncthreads();   // the page and the per-key slots in LDS are free for the next page
+  jp = nj;
   }
 }
 
@@ -2445,8 +2475,11 @@ int launch_gram(const GramArgs& a, int L, hipStream_t st) {
     }
   }
   if constexpr (T::bytes == 4 && !RAW) {
-    if (a.BS <= kPage32Rows && a.BS % 32 == 0) {
-      const size_t smem = (size_t)kPage32Rows * ROWF * 4 + (size_t)kPage32Rows * (8 + 8 + 4 + 4 * 4);
+    if (a.BS <= kPage32Rows && a.BS % 32 == 0 && a.NB <= 1024) {
+      // one workgroup per (layer, sequence, kv head) row
+      grid = dim3((unsigned)((int64_t)L * a.B * a.Hkv));
+      const size_t smem = (size_t)kPage32Rows * ROWF * 4 + (size_t)kPage32Rows * (8 + 8 + 4 + 4 * 4) +
+                          sizeof(int) * a.NB;
       if (hipFuncSetAttribute((const void*)gram_page_f32_kernel,
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess) {
         zp_set_error("redundancy: cannot reserve %zu bytes of LDS", smem);
