@@ -12,8 +12,9 @@
 //   gram_kernel        fp32 caches, both variants: v_mfma_f32_32x32x2_f32 on keys divided by
 //                      their cache-dtype norm in fp32 (the reference's arithmetic), full
 //                      matrix, a wave owns 32 rows for all columns.
-//   gram_page_f32_kernel  fp32 caches, lightning, pages of at most 256 keys: the normalised page
-//                      resident in LDS, one barrier, both operands read from that copy.
+//   gram_page_f32_kernel  fp32 caches, lightning, pages of at most 256 keys: a workgroup walks the
+//                      pages of a row; the normalised page resident in LDS, one barrier, both
+//                      operands read from that copy, the next page requested under the tiles.
 //   gram_split_kernel  16-bit caches, lightning with pages above 256 keys: normalised keys
 //                      split into two bf16 planes, three MFMAs per k-step, full matrix.
 //   gram_page_kernel   16-bit caches, lightning: a workgroup walks the pages of one (layer,
@@ -21,7 +22,7 @@
 //                      the matrix cores, 1/norm factors on the accumulators, every pair of key
 //                      blocks once, the summed key as a product over the keys, the next page
 //                      requested while a page's row sums are finished.
-//   raw_prep_kernel, gram_raw_kernel, raw_claim_value_kernel, raw_chain_kernel
+//   raw_prep_kernel, gram_raw_wide_kernel / gram_raw_kernel, raw_claim_value_kernel, raw_chain_kernel
 //                      16-bit caches, raw: the same over the pages of a sequence, the row sums
 //                      accumulated in the cache dtype chunk by chunk as the reference does.
 //   red_softmax_kernel claim corrections of the raw variant and the softmax of both.
@@ -577,10 +578,11 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
 }
 
 // ------------------------------------------------------------------ fp32 caches, lightning, whole page in LDS
-// One workgroup per (layer, sequence, head, page) of at most 256 keys: the page is loaded once
-// with coalesced 16-byte loads, normalised on the way into LDS (132 KB), and after ONE barrier
-// every wave multiplies its 32 rows (A operand read from the same LDS copy) with its share of the
-// column blocks (every unordered pair of blocks once): no tile pipeline, no strided row loads.
+// Pages of at most 256 keys; one workgroup per (layer, sequence, head) row walks the row's pages:
+// a page is loaded once with coalesced 16-byte loads into registers (requested under the tiles of
+// the page before), normalised on the way into LDS (132 KB), and after ONE barrier every wave
+// multiplies its 32 rows (A operand read from the same LDS copy) with its share of the column
+// blocks (every unordered pair of blocks once): no tile pipeline, no strided row loads.
 constexpr int kPage32Rows = 256;
 constexpr int kPage32Threads = 512;
 __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs p) {
