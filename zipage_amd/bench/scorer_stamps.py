@@ -40,7 +40,7 @@ def main():
     _, S, W, Hq, _ = q.shape
     NB = enc.shape[1]
     lib = _lib.load()
-    need = lib.zp_attention_score_workspace(L, B, NB, BS, Hkv, Hq, W)
+    need = lib.zp_attention_score_workspace_for(L, B, NB, BS, Hkv, Hq, W, _lib.dtype_tag(k))
     RB = (W * (Hq // Hkv) + 31) // 32
     units = L * B * Hkv * RB
     ws = torch.zeros(need + units * 64, dtype=torch.uint8, device=k.device)
