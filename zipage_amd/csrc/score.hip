@@ -129,6 +129,12 @@ __device__ __forceinline__ float vmax(float a, float b) {
   asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
   return d;
 }
+__device__ __forceinline__ float vmax3(float a, float b, float c) {
+  float d;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+  return d;
+}
+__device__ __forceinline__ float vmax4(float a, float b, float c, float d) { return vmax(vmax3(a, b, c), d); }
 __device__ __forceinline__ float vmax_neg(float a, float b) {  // max(a, -b)
   float d;
   asm("v_max_f32 %0, %1, -%2" : "=v"(d) : "v"(a), "v"(b));
@@ -401,7 +407,7 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
               }
               if (sgn > 0.f) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) run[r] = vmax(vmax(run[r], accA[r]), accB[r]);
+                for (int r = 0; r < 16; ++r) run[r] = vmax3(run[r], accA[r], accB[r]);
               } else {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) run[r] = vmax_neg(vmax_neg(run[r], accA[r]), accB[r]);
@@ -516,7 +522,7 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
                   float q4[4];
 #pragma unroll
                   for (int q = 0; q < 4; ++q)
-                    q4[q] = vmax(vmax(pv[4 * q], pv[4 * q + 1]), vmax(pv[4 * q + 2], pv[4 * q + 3]));
+                    q4[q] = vmax4(pv[4 * q], pv[4 * q + 1], pv[4 * q + 2], pv[4 * q + 3]);
                   if (Gp >= 8) {
 #pragma unroll
                     for (int q = 0; q < 4; ++q) q4[q] = vmax(q4[q], lane_xor32(q4[q]));
@@ -541,7 +547,7 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
                       red = rmaxV ? vmax(q4[0], q4[2]) : q4[0] + q4[2];
                     }
                   } else {
-                    red = rmaxV ? vmax(vmax(q4[0], q4[1]), vmax(q4[2], q4[3]))
+                    red = rmaxV ? vmax4(q4[0], q4[1], q4[2], q4[3])
                                        : (q4[0] + q4[1]) + (q4[2] + q4[3]);
                   }
                 } else {
@@ -557,8 +563,7 @@ __global__ __launch_bounds__(kThreads, (T::bytes == 2 ? kOcc16 : 1)) void score_
                       t8[q] = rmaxV ? vmax(pv[2 * q], pv[2 * q + 1]) : pv[2 * q] + pv[2 * q + 1];
                   }
                   if (rmaxV) {
-                    red = vmax(vmax(vmax(t8[0], t8[1]), vmax(t8[2], t8[3])),
-                                vmax(vmax(t8[4], t8[5]), vmax(t8[6], t8[7])));
+                    red = vmax3(vmax3(t8[0], t8[1], t8[2]), vmax3(t8[3], t8[4], t8[5]), vmax(t8[6], t8[7]));
                   } else {
                     red = ((t8[0] + t8[1]) + (t8[2] + t8[3])) + ((t8[4] + t8[5]) + (t8[6] + t8[7]));
                   }
@@ -776,7 +781,7 @@ __device__ __forceinline__ float group_window_reduce(float (&pv)[16], int Gp, bo
     float q4[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-      q4[q] = vmax(vmax(pv[4 * q], pv[4 * q + 1]), vmax(pv[4 * q + 2], pv[4 * q + 3]));
+      q4[q] = vmax4(pv[4 * q], pv[4 * q + 1], pv[4 * q + 2], pv[4 * q + 3]);
     if (Gp >= 8) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) q4[q] = vmax(q4[q], lane_xor32(q4[q]));
@@ -801,7 +806,7 @@ __device__ __forceinline__ float group_window_reduce(float (&pv)[16], int Gp, bo
         red = rmaxV ? vmax(q4[0], q4[2]) : q4[0] + q4[2];
       }
     } else {
-      red = rmaxV ? vmax(vmax(q4[0], q4[1]), vmax(q4[2], q4[3])) : (q4[0] + q4[1]) + (q4[2] + q4[3]);
+      red = rmaxV ? vmax4(q4[0], q4[1], q4[2], q4[3]) : (q4[0] + q4[1]) + (q4[2] + q4[3]);
     }
   } else {
     float t8[8];
@@ -815,7 +820,7 @@ __device__ __forceinline__ float group_window_reduce(float (&pv)[16], int Gp, bo
       for (int q = 0; q < 8; ++q) t8[q] = rmaxV ? vmax(pv[2 * q], pv[2 * q + 1]) : pv[2 * q] + pv[2 * q + 1];
     }
     if (rmaxV) {
-      red = vmax(vmax(vmax(t8[0], t8[1]), vmax(t8[2], t8[3])), vmax(vmax(t8[4], t8[5]), vmax(t8[6], t8[7])));
+      red = vmax3(vmax3(t8[0], t8[1], t8[2]), vmax3(t8[3], t8[4], t8[5]), vmax(t8[6], t8[7]));
     } else {
       red = ((t8[0] + t8[1]) + (t8[2] + t8[3])) + ((t8[4] + t8[5]) + (t8[6] + t8[7]));
     }
@@ -1364,12 +1369,12 @@ __global__ __launch_bounds__(kThreads, 2) void score_resident_f32_kernel(ScoreAr
       // groups of 8 / 16 rows span two / four lane groups
       float red;
       if (GpV == 1) {
-        red = rmaxV ? vmax(vmax(pv[0], pv[1]), vmax(pv[2], pv[3])) : (pv[0] + pv[1]) + (pv[2] + pv[3]);
+        red = rmaxV ? vmax4(pv[0], pv[1], pv[2], pv[3]) : (pv[0] + pv[1]) + (pv[2] + pv[3]);
       } else if (GpV == 2) {
         const float g0 = vmax(pv[0], pv[1]), g1 = vmax(pv[2], pv[3]);
         red = rmaxV ? vmax(g0, g1) : g0 + g1;
       } else {
-        red = vmax(vmax(pv[0], pv[1]), vmax(pv[2], pv[3]));
+        red = vmax4(pv[0], pv[1], pv[2], pv[3]);
       }
       {
         const float o = lane_xor16(red);
