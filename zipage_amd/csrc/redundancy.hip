@@ -577,6 +577,40 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
   }
 }
 
+// ------------------------------------------------------------------ fp32 products on the fp16 matrix cores
+// A normalised key element x (|x| <= 1) is scaled by 2^12 and written as two fp16 numbers,
+// h1 = fp16(x') and h2 = fp16(x' - h1), both rounded to nearest: x' - h1 is exact in fp32 (13
+// bits), so |x' - h1 - h2| <= 2^-24 |x'|, what rounding a real number to fp32 loses; the scale
+// keeps h2 out of fp16's subnormal range for every element that matters (|x| >= 2^-14) and the
+// largest scaled element (4096) far below fp16's maximum.  The products h1.g1, h1.g2, h2.g1 are
+// exact in the fp32 accumulator, h2.g2 (<= 2^-24 |x||y|) is left out, and the 2^24 of the two
+// scales comes off the result exactly.  Three v_mfma_f32_32x32x16_f16 (8 passes each, 16 k) replace eight
+// v_mfma_f32_32x32x2_f32 (16 passes each): 3/16 of the matrix-core time at fp32-grade accuracy, and the
+// two planes take the LDS bytes of the fp32 element they replace.
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+constexpr float kPlaneScale = 4096.f;                 // 2^12 per operand
+constexpr float kPlaneUnscale = 1.f / (4096.f * 4096.f);
+constexpr int KSH = kDmax / 16;                       // k-steps of the 16-bit instructions over a key row
+constexpr int kPlaneBytes = kDmax * 2;                // one plane of one LDS row; the row keeps ROWF * 4 bytes
+__device__ __forceinline__ void split_planes(const float4 e, f16x4_t& h1, f16x4_t& h2) {
+  const f32x2_t a = {e.x, e.y}, b = {e.z, e.w};
+  const f16x2_t a1 = __builtin_convertvector(a, f16x2_t), b1 = __builtin_convertvector(b, f16x2_t);
+  const f32x2_t ar = {e.x - (float)a1[0], e.y - (float)a1[1]}, br = {e.z - (float)b1[0], e.w - (float)b1[1]};
+  const f16x2_t a2 = __builtin_convertvector(ar, f16x2_t), b2 = __builtin_convertvector(br, f16x2_t);
+  h1 = f16x4_t{a1[0], a1[1], b1[0], b1[1]};
+  h2 = f16x4_t{a2[0], a2[1], b2[0], b2[1]};
+}
+__device__ __forceinline__ f32x16_t mma_planes(const f16x8_t a1, const f16x8_t a2, const f16x8_t b1,
+                                               const f16x8_t b2, f32x16_t acc) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b1, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b2, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b1, acc, 0, 0, 0);
+  return acc;
+}
+
 // ------------------------------------------------------------------ fp32 caches, lightning, whole page in LDS
 // Pages of at most 256 keys; one workgroup per (layer, sequence, head) row walks the row's pages:
 // a page is loaded once with coalesced 16-byte loads into registers (requested under the tiles of
@@ -660,8 +694,12 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
       const float4 e = raw[it];
       float ss = (e.x * e.x + e.y * e.y) + (e.z * e.z + e.w * e.w);
       ss = pieces_sum<PIECES>(ss);
-      const float rn = __builtin_amdgcn_rcpf(fmaxf(__builtin_amdgcn_sqrtf(ss), p.eps));
-      *(float4*)(kpl + row * ROWF + piece * 4) = make_float4(e.x * rn, e.y * rn, e.z * rn, e.w * rn);
+      const float rn = __builtin_amdgcn_rcpf(fmaxf(__builtin_amdgcn_sqrtf(ss), p.eps)) * kPlaneScale;
+      f16x4_t h1, h2;
+      split_planes(make_float4(e.x * rn, e.y * rn, e.z * rn, e.w * rn), h1, h2);
+      char* dst = (char*)(kpl + row * ROWF) + piece * 8;
+      *(f16x4_t*)dst = h1;
+      *(f16x4_t*)(dst + kPlaneBytes) = h2;
     }
   }
   __syncthreads();
@@ -678,14 +716,14 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
   const int nrb = p.BS / 32;
   if (wave < nrb) {
     const int rb = wave;
-    float afrag[KS];
+    // lane (col, half) holds elements 16 s + 8 half .. + 7 of key rb * 32 + col for k-step s
+    f16x8_t a1[KSH], a2[KSH];
     {
-      const float4* a4 = (const float4*)(kpl + (rb * 32 + col) * ROWF + 4 * half);
+      const char* ar = (const char*)(kpl + (rb * 32 + col) * ROWF) + 16 * half;
 #pragma unroll
-      for (int j4 = 0; j4 < KS / 4; ++j4) {
-        const float4 av = a4[2 * j4];
-        afrag[4 * j4 + 0] = av.x; afrag[4 * j4 + 1] = av.y;
-        afrag[4 * j4 + 2] = av.z; afrag[4 * j4 + 3] = av.w;
+      for (int s = 0; s < KSH; ++s) {
+        a1[s] = *(const f16x8_t*)(ar + 32 * s);
+        a2[s] = *(const f16x8_t*)(ar + kPlaneBytes + 32 * s);
       }
     }
     float rsum[16], cval[16];
@@ -699,22 +737,18 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
       f32x16_t acc;
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-      const float4* b4 = (const float4*)(kpl + (cb * 32 + col) * ROWF + 4 * half);
+      const char* br = (const char*)(kpl + (cb * 32 + col) * ROWF) + 16 * half;
 #pragma unroll
-      for (int j4 = 0; j4 < KS / 4; ++j4) {
-        const float4 bv = b4[2 * j4];
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 0], bv.x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 1], bv.y, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 2], bv.z, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 3], bv.w, acc, 0, 0, 0);
-      }
+      for (int s = 0; s < KSH; ++s)
+        acc = mma_planes(a1[s], a2[s], *(const f16x8_t*)(br + 32 * s),
+                         *(const f16x8_t*)(br + kPlaneBytes + 32 * s), acc);
       const int cslot = cb * 32 + col;
       float csum = 0.f, rv = 0.f;     // column side: sum over this lane's rows, last row over the threshold
       int rlast = -1;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-        float sv = acc[r];
+        float sv = acc[r] * kPlaneUnscale;
         if (rslot == cslot) sv = 0.f;
         rsum[r] += sv;
         csum += sv;
