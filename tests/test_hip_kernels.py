@@ -563,6 +563,47 @@ def test_raw_redundancy_page_counts(dev, dtype, nb_choices):
         _ulp_close(gr, wr, dtype, ulps=4)
 
 
+@pytest.mark.parametrize("variant", ["lightning", "raw"])
+def test_fp32_redundancy_products_are_fp32_grade(dev, variant):
+    """fp32 caches: the key products run as two fp16 planes per operand on the 16-bit matrix
+    instructions.  With no claims (threshold 2) the logits are plain sums of cosines, which a
+    float64 evaluation gives to 1e-15: the distance to it must be what fp32 arithmetic leaves.
+    Measured: mean 1.1e-6 / 2.4e-6 (lightning / raw), max 4.9e-6 / 9.5e-6, against 0.9e-6 / 1.5e-6
+    and 4.1e-6 / 9.6e-6 with fp32 matrix instructions; a two-plane bf16 split would be 16-64
+    times further away, TF32 a thousand times.  Elements of very different sizes inside a key
+    (1e-5 .. 1) and keys of very different norms exercise the planes' scale."""
+    from zipage_amd import kernel as K
+    s = _setup(97, torch.float32, L=1, B=2, Hkv=2, Hq=2, nb_choices=(2, 3), num_pages=12)
+    g = torch.Generator().manual_seed(31)
+    k = s["k"].float()
+    k = k * torch.logspace(-5, 0, 128).view(1, 1, 1, 1, 128)[..., torch.randperm(128, generator=g)]
+    k = (k * torch.logspace(-3, 3, k.shape[2]).view(1, 1, -1, 1, 1)).contiguous()
+    fn = K.lightning_redudancy_score if variant == "lightning" else K.raw_redudancy_score
+    gl, _ = fn(k.to(dev), s["enc"].to(dev), threshold=2.0, temperature=0.4, return_logits=True)
+    L, _, BS, Hkv, D = k.shape
+    gl = gl.cpu().double().view(L, len(s["tables"]), Hkv, -1, BS)
+    worst, total, count = 0.0, 0.0, 0
+    for b, table in enumerate(s["tables"]):
+        pages = [(j, pid) for j, pid in enumerate(table) if pid >= 0]
+        for h in range(Hkv):
+            x = torch.cat([k[0, pid, :, h].double() for _, pid in pages])
+            x = x / x.norm(dim=-1, keepdim=True).clamp_min(1e-6)
+            sim = x @ x.T
+            sim.fill_diagonal_(0.0)
+            if variant == "lightning":     # only pairs inside a page
+                blk = torch.block_diag(*[torch.ones(BS, BS, dtype=torch.float64)] * len(pages))
+                sim = sim * blk
+            want = sim.sum(1)
+            got = torch.cat([gl[0, b, h, j] for j, _ in pages])
+            err = (got - want).abs()
+            worst = max(worst, err.max().item())
+            total += err.sum().item()
+            count += err.numel()
+    print(f"fp32 {variant}: row sums against float64: max {worst:.2e}, mean {total / count:.2e}")
+    max_bound, mean_bound = (1.5e-5, 3e-6) if variant == "lightning" else (3e-5, 7e-6)
+    assert worst < max_bound and total / count < mean_bound
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_raw_redundancy(dev, dtype):
     from zipage_amd.kernel import raw_redudancy_score

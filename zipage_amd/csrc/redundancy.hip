@@ -368,6 +368,40 @@ __global__ __launch_bounds__(NW * 64) void gram_kernel(GramArgs p) {
   }
 }
 
+// ------------------------------------------------------------------ fp32 products on the fp16 matrix cores
+// A normalised key element x (|x| <= 1) is scaled by 2^12 and written as two fp16 numbers,
+// h1 = fp16(x') and h2 = fp16(x' - h1), both rounded to nearest: x' - h1 is exact in fp32 (13
+// bits), so |x' - h1 - h2| <= 2^-24 |x'|, what rounding a real number to fp32 loses; the scale
+// keeps h2 out of fp16's subnormal range for every element that matters (|x| >= 2^-14) and the
+// largest scaled element (4096) far below fp16's maximum.  The products h1.g1, h1.g2, h2.g1 are
+// exact in the fp32 accumulator, h2.g2 (<= 2^-24 |x||y|) is left out, and the 2^24 of the two
+// scales comes off the result exactly.  Three v_mfma_f32_32x32x16_f16 (8 passes each, 16 k) replace eight
+// v_mfma_f32_32x32x2_f32 (16 passes each): 3/16 of the matrix-core time at fp32-grade accuracy, and the
+// two planes take the LDS bytes of the fp32 element they replace.
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+constexpr float kPlaneScale = 4096.f;                 // 2^12 per operand
+constexpr float kPlaneUnscale = 1.f / (4096.f * 4096.f);
+constexpr int KSH = kDmax / 16;                       // k-steps of the 16-bit instructions over a key row
+constexpr int kPlaneBytes = kDmax * 2;                // one plane of one LDS row; the row keeps ROWF * 4 bytes
+__device__ __forceinline__ void split_planes(const float4 e, f16x4_t& h1, f16x4_t& h2) {
+  const f32x2_t a = {e.x, e.y}, b = {e.z, e.w};
+  const f16x2_t a1 = __builtin_convertvector(a, f16x2_t), b1 = __builtin_convertvector(b, f16x2_t);
+  const f32x2_t ar = {e.x - (float)a1[0], e.y - (float)a1[1]}, br = {e.z - (float)b1[0], e.w - (float)b1[1]};
+  const f16x2_t a2 = __builtin_convertvector(ar, f16x2_t), b2 = __builtin_convertvector(br, f16x2_t);
+  h1 = f16x4_t{a1[0], a1[1], b1[0], b1[1]};
+  h2 = f16x4_t{a2[0], a2[1], b2[0], b2[1]};
+}
+__device__ __forceinline__ f32x16_t mma_planes(const f16x8_t a1, const f16x8_t a2, const f16x8_t b1,
+                                               const f16x8_t b2, f32x16_t acc) {
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b1, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b2, acc, 0, 0, 0);
+  acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b1, acc, 0, 0, 0);
+  return acc;
+}
+
 // ------------------------------------------------------------------ fp32 caches, raw, every pair of pages once
 // One workgroup per (layer, sequence, head, valid page a), pages of at most 256 keys.  The
 // similarity matrix of a sequence is symmetric, so page a multiplies its rows only with the pages
@@ -450,41 +484,47 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
       Unpack<T>::run(pre[i], e);
       float ss = (e[0] * e[0] + e[1] * e[1]) + (e[2] * e[2] + e[3] * e[3]);
       ss = pieces_sum<PIECES>(ss);
-      const float rn = __builtin_amdgcn_rcpf(fmaxf(__builtin_amdgcn_sqrtf(ss), p.eps));
-      if (st_piece < dpieces)
-        *(float4*)(buf + row * ROWF + st_piece * 4) = make_float4(e[0] * rn, e[1] * rn, e[2] * rn, e[3] * rn);
+      const float rn = __builtin_amdgcn_rcpf(fmaxf(__builtin_amdgcn_sqrtf(ss), p.eps)) * kPlaneScale;
+      if (st_piece < dpieces) {
+        f16x4_t h1, h2;
+        split_planes(make_float4(e[0] * rn, e[1] * rn, e[2] * rn, e[3] * rn), h1, h2);
+        char* dst = (char*)(buf + row * ROWF) + st_piece * 8;
+        *(f16x4_t*)dst = h1;
+        *(f16x4_t*)(dst + kPlaneBytes) = h2;
+      }
     }
   };
 
   const int row_blocks = p.BS / 32;
   const int rb = wave;
   const bool active = rb < row_blocks;
-  // A fragments: this lane's key row of page a, normalised; k-step 4j + i of wave half `half` takes
-  // element 8j + 4 half + i (the same order as the B operand's 16-byte LDS reads)
-  float afrag[KS];
+  // A fragments: this lane's key row of page a, normalised and split; k-step s of wave half
+  // `half` takes elements 16 s + 8 half .. + 7 (pieces 4 s + 2 half and the next one), the same
+  // order as the B operand's 16-byte LDS reads
+  f16x8_t a1[KSH], a2[KSH];
   {
     const int slot = (active ? rb : 0) * 32 + col;
     const char* src = kbase + (int64_t)rpid * p.k_sp * 4 + (int64_t)slot * k_row;
+    float4 mine[2 * KSH];
     float ss = 0.f;
 #pragma unroll
     for (int pc = 0; pc < PIECES; ++pc) {
-      float e[4];
-      vec16 v = vec16{0u, 0u, 0u, 0u};
-      if (pc < dpieces) v = *(const vec16*)(src + pc * 16);
-      Unpack<T>::run(v, e);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) ss += e[q] * e[q];
-      if ((pc & 1) == 0) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) afrag[(pc >> 1) * 4 + q] = e[q];
-      } else if (half) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) afrag[(pc >> 1) * 4 + q] = e[q];
-      }
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (pc < dpieces) v = *(const float4*)(src + pc * 16);
+      ss += (v.x * v.x + v.y * v.y) + (v.z * v.z + v.w * v.w);
+      if (((pc >> 1) & 1) == 0) mine[(pc >> 2) * 2 + (pc & 1)] = v;
+      else if (half) mine[(pc >> 2) * 2 + (pc & 1)] = v;
     }
-    const float rn = __builtin_amdgcn_rcpf(fmaxf(__builtin_amdgcn_sqrtf(ss), p.eps));
+    const float rn = active ? __builtin_amdgcn_rcpf(fmaxf(__builtin_amdgcn_sqrtf(ss), p.eps)) * kPlaneScale : 0.f;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) afrag[s] = active ? afrag[s] * rn : 0.f;
+    for (int s = 0; s < KSH; ++s) {
+      f16x4_t l1, l2, u1, u2;
+      const float4 lo = mine[2 * s], up = mine[2 * s + 1];
+      split_planes(make_float4(lo.x * rn, lo.y * rn, lo.z * rn, lo.w * rn), l1, l2);
+      split_planes(make_float4(up.x * rn, up.y * rn, up.z * rn, up.w * rn), u1, u2);
+      a1[s] = f16x8_t{l1[0], l1[1], l1[2], l1[3], u1[0], u1[1], u1[2], u1[3]};
+      a2[s] = f16x8_t{l2[0], l2[1], l2[2], l2[3], u2[0], u2[1], u2[2], u2[3]};
+    }
   }
   float rsum[16], cval[16];
   int ccol[16];
@@ -521,21 +561,17 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
         f32x16_t acc;
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-        const float4* b4 = (const float4*)(cur + (st * 32 + col) * ROWF + 4 * half);
+        const char* br = (const char*)(cur + (st * 32 + col) * ROWF) + 16 * half;
 #pragma unroll
-        for (int j4 = 0; j4 < KS / 4; ++j4) {
-          const float4 bv = b4[2 * j4];
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 0], bv.x, acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 1], bv.y, acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 2], bv.z, acc, 0, 0, 0);
-          acc = __builtin_amdgcn_mfma_f32_32x32x2f32(afrag[4 * j4 + 3], bv.w, acc, 0, 0, 0);
-        }
+        for (int s = 0; s < KSH; ++s)
+          acc = mma_planes(a1[s], a2[s], *(const f16x8_t*)(br + 32 * s),
+                           *(const f16x8_t*)(br + kPlaneBytes + 32 * s), acc);
         const int cslot = toff + st * 32 + col;
         const int cidx = jc * p.BS + cslot;   // logical index of this lane's column key
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-          float sv = acc[r];
+          float sv = acc[r] * kPlaneUnscale;
           if (d == 0 && rslot == cslot) sv = 0.f;
           rsum[r] += sv;
           csum += sv;
@@ -575,40 +611,6 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
         atomicMax(&ws_claim[oi], ((unsigned long long)(unsigned)(c + 1) << 32) | __float_as_uint(v));
     }
   }
-}
-
-// ------------------------------------------------------------------ fp32 products on the fp16 matrix cores
-// A normalised key element x (|x| <= 1) is scaled by 2^12 and written as two fp16 numbers,
-// h1 = fp16(x') and h2 = fp16(x' - h1), both rounded to nearest: x' - h1 is exact in fp32 (13
-// bits), so |x' - h1 - h2| <= 2^-24 |x'|, what rounding a real number to fp32 loses; the scale
-// keeps h2 out of fp16's subnormal range for every element that matters (|x| >= 2^-14) and the
-// largest scaled element (4096) far below fp16's maximum.  The products h1.g1, h1.g2, h2.g1 are
-// exact in the fp32 accumulator, h2.g2 (<= 2^-24 |x||y|) is left out, and the 2^24 of the two
-// scales comes off the result exactly.  Three v_mfma_f32_32x32x16_f16 (8 passes each, 16 k) replace eight
-// v_mfma_f32_32x32x2_f32 (16 passes each): 3/16 of the matrix-core time at fp32-grade accuracy, and the
-// two planes take the LDS bytes of the fp32 element they replace.
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
-typedef __attribute__((ext_vector_type(4))) _Float16 f16x4_t;
-typedef __attribute__((ext_vector_type(2))) _Float16 f16x2_t;
-typedef __attribute__((ext_vector_type(2))) float f32x2_t;
-constexpr float kPlaneScale = 4096.f;                 // 2^12 per operand
-constexpr float kPlaneUnscale = 1.f / (4096.f * 4096.f);
-constexpr int KSH = kDmax / 16;                       // k-steps of the 16-bit instructions over a key row
-constexpr int kPlaneBytes = kDmax * 2;                // one plane of one LDS row; the row keeps ROWF * 4 bytes
-__device__ __forceinline__ void split_planes(const float4 e, f16x4_t& h1, f16x4_t& h2) {
-  const f32x2_t a = {e.x, e.y}, b = {e.z, e.w};
-  const f16x2_t a1 = __builtin_convertvector(a, f16x2_t), b1 = __builtin_convertvector(b, f16x2_t);
-  const f32x2_t ar = {e.x - (float)a1[0], e.y - (float)a1[1]}, br = {e.z - (float)b1[0], e.w - (float)b1[1]};
-  const f16x2_t a2 = __builtin_convertvector(ar, f16x2_t), b2 = __builtin_convertvector(br, f16x2_t);
-  h1 = f16x4_t{a1[0], a1[1], b1[0], b1[1]};
-  h2 = f16x4_t{a2[0], a2[1], b2[0], b2[1]};
-}
-__device__ __forceinline__ f32x16_t mma_planes(const f16x8_t a1, const f16x8_t a2, const f16x8_t b1,
-                                               const f16x8_t b2, f32x16_t acc) {
-  acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a2, b1, acc, 0, 0, 0);
-  acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b2, acc, 0, 0, 0);
-  acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b1, acc, 0, 0, 0);
-  return acc;
 }
 
 // ------------------------------------------------------------------ fp32 caches, lightning, whole page in LDS
