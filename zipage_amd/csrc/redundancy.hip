@@ -401,6 +401,15 @@ __device__ __forceinline__ f32x16_t mma_planes(const f16x8_t a1, const f16x8_t a
   acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(a1, b1, acc, 0, 0, 0);
   return acc;
 }
+// largest of a lane's sixteen tile entries (claims are rare: one maximum per lane and a ballot
+// decide whether a tile has any entry over the threshold)
+__device__ __forceinline__ float tile_lane_max(const f32x16_t& acc) {
+  float m[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+    m[q] = __builtin_fmaxf(__builtin_fmaxf(acc[4 * q], acc[4 * q + 1]), __builtin_fmaxf(acc[4 * q + 2], acc[4 * q + 3]));
+  return __builtin_fmaxf(__builtin_fmaxf(m[0], m[1]), __builtin_fmaxf(m[2], m[3]));
+}
 
 // ------------------------------------------------------------------ fp32 caches, raw, every pair of pages once
 // One workgroup per (layer, sequence, head, valid page a), pages of at most 256 keys.  The
@@ -530,6 +539,8 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
   int ccol[16];
 #pragma unroll
   for (int r = 0; r < 16; ++r) { rsum[r] = 0.f; cval[r] = 0.f; ccol[r] = -1; }
+  const float thr_s = p.threshold * (kPlaneScale * kPlaneScale);
+  bool wave_claims = false;       // any tile of this wave with an entry over the threshold (uniform)
 
   // the column sums of tile t are complete after the barrier that ends it: the waves' shares are
   // added in wave order and stored while tile t+1 is being multiplied
@@ -541,7 +552,7 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
 #pragma unroll
     for (int w2 = 1; w2 < kSymWaves; ++w2) v += pt[w2 * TN + tid];
     const int jc = vidx[col_page(d)];
-    p.ws_chunk[(int64_t)(d - 1) * n_keys + obase + (int64_t)jc * p.BS + toff + tid] = v;
+    p.ws_chunk[(int64_t)(d - 1) * n_keys + obase + (int64_t)jc * p.BS + toff + tid] = v * kPlaneUnscale;
   };
 
   if (ntiles > 0) { issue_loads(0); commit_loads(kbuf0); }
@@ -566,26 +577,39 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
         for (int s = 0; s < KSH; ++s)
           acc = mma_planes(a1[s], a2[s], *(const f16x8_t*)(br + 32 * s),
                            *(const f16x8_t*)(br + kPlaneBytes + 32 * s), acc);
+        // sums, claim values and the threshold stay in the planes' scale (a power of two: the
+        // same bits come out when it is taken off at the end)
         const int cslot = toff + st * 32 + col;
         const int cidx = jc * p.BS + cslot;   // logical index of this lane's column key
+        if (d == 0) {     // the page against itself: a key is not its own neighbour
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-          float sv = acc[r] * kPlaneUnscale;
-          if (d == 0 && rslot == cslot) sv = 0.f;
-          rsum[r] += sv;
-          csum += sv;
-          const bool over = sv > p.threshold;
-          if (over && cidx > ccol[r]) { ccol[r] = cidx; cval[r] = sv; }
-          if (over) { rlast = rslot; rv = sv; }   // rslot grows with r inside a lane
+          for (int r = 0; r < 16; ++r)
+            if (rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3) == cslot) acc[r] = 0.f;
         }
-        if (d != 0) {
-          const int orl = lane_xor32(rlast);
-          const float orv = lane_xor32(rv);
-          if (orl > rlast) { rlast = orl; rv = orv; }
-          if (half == 0 && rlast >= 0)   // rare: the column key's claim candidate among page a's rows
-            atomicMax(&ws_claim[obase + cidx],
-                      ((unsigned long long)(unsigned)(jp * p.BS + rlast + 1) << 32) | __float_as_uint(rv));
+        const bool any_over = __builtin_amdgcn_ballot_w64(tile_lane_max(acc) > thr_s) != 0ull;
+        wave_claims |= any_over;
+        if (!any_over) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) { rsum[r] += acc[r]; csum += acc[r]; }
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+            const float sv = acc[r];
+            rsum[r] += sv;
+            csum += sv;
+            const bool over = sv > thr_s;
+            if (over && cidx > ccol[r]) { ccol[r] = cidx; cval[r] = sv; }
+            if (over) { rlast = rslot; rv = sv; }   // rslot grows with r inside a lane
+          }
+          if (d != 0) {
+            const int orl = lane_xor32(rlast);
+            const float orv = lane_xor32(rv);
+            if (orl > rlast) { rlast = orl; rv = orv; }
+            if (half == 0 && rlast >= 0)   // the column key's claim candidate among page a's rows
+              atomicMax(&ws_claim[obase + cidx], ((unsigned long long)(unsigned)(jp * p.BS + rlast + 1) << 32) |
+                                                     __float_as_uint(rv * kPlaneUnscale));
+          }
         }
       }
       if (d != 0) {
@@ -603,12 +627,12 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
     float sv = half_sum(rsum[r]);
     int c = ccol[r];
     float v = cval[r];
-    last_claim_reduce(c, v);
+    if (wave_claims) last_claim_reduce(c, v);
     if (active && col == 0) {
       const int64_t oi = obase + (int64_t)jp * p.BS + rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-      p.ws_sum[oi] = sv;
+      p.ws_sum[oi] = sv * kPlaneUnscale;
       if (c >= 0)
-        atomicMax(&ws_claim[oi], ((unsigned long long)(unsigned)(c + 1) << 32) | __float_as_uint(v));
+        atomicMax(&ws_claim[oi], ((unsigned long long)(unsigned)(c + 1) << 32) | __float_as_uint(v * kPlaneUnscale));
     }
   }
 }
@@ -733,6 +757,8 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
 #pragma unroll
     for (int r = 0; r < 16; ++r) { rsum[r] = 0.f; cval[r] = 0.f; ccol[r] = -1; }
     const int nd = nrb / 2 + (((nrb & 1) || rb < nrb / 2) ? 1 : 0);   // distances 0 .. nd-1
+    const float thr_s = p.threshold * (kPlaneScale * kPlaneScale);
+    bool wave_claims = false;     // any tile of this wave with an entry over the threshold (uniform)
 #pragma unroll 1
     for (int d = 0; d < nd; ++d) {
       const int cb = rb + d < nrb ? rb + d : rb + d - nrb;
@@ -744,28 +770,44 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
       for (int s = 0; s < KSH; ++s)
         acc = mma_planes(a1[s], a2[s], *(const f16x8_t*)(br + 32 * s),
                          *(const f16x8_t*)(br + kPlaneBytes + 32 * s), acc);
+      // sums, claim values and the threshold stay in the planes' scale (a power of two: the same
+      // bits come out when it is taken off at the end)
       const int cslot = cb * 32 + col;
+      if (d == 0) {     // the block against itself: a key is not its own neighbour
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          if (rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3) == cslot) acc[r] = 0.f;
+      }
+      const bool any_over = __builtin_amdgcn_ballot_w64(tile_lane_max(acc) > thr_s) != 0ull;
+      wave_claims |= any_over;
       float csum = 0.f, rv = 0.f;     // column side: sum over this lane's rows, last row over the threshold
       int rlast = -1;
+      if (!any_over) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-        float sv = acc[r] * kPlaneUnscale;
-        if (rslot == cslot) sv = 0.f;
-        rsum[r] += sv;
-        csum += sv;
-        const bool over = sv > p.threshold;
-        if (over && cslot > ccol[r]) { ccol[r] = cslot; cval[r] = sv; }
-        if (over) { rlast = rslot; rv = sv; }     // rslot grows with r inside a lane
+        for (int r = 0; r < 16; ++r) { rsum[r] += acc[r]; csum += acc[r]; }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+          const float sv = acc[r];
+          rsum[r] += sv;
+          csum += sv;
+          const bool over = sv > thr_s;
+          if (over && cslot > ccol[r]) { ccol[r] = cslot; cval[r] = sv; }
+          if (over) { rlast = rslot; rv = sv; }     // rslot grows with r inside a lane
+        }
       }
       if (d != 0) {
         csum += lane_xor32(csum);
-        if (half == 0) l_csum[(d - 1) * kPage32Rows + cslot] = csum;
-        const int orl = lane_xor32(rlast);
-        const float orv = lane_xor32(rv);
-        if (orl > rlast) { rlast = orl; rv = orv; }
-        if (half == 0 && rlast >= 0)
-          atomicMax(&l_claim[cslot], ((unsigned long long)(unsigned)(rlast + 1) << 32) | __float_as_uint(rv));
+        if (half == 0) l_csum[(d - 1) * kPage32Rows + cslot] = csum * kPlaneUnscale;
+        if (any_over) {
+          const int orl = lane_xor32(rlast);
+          const float orv = lane_xor32(rv);
+          if (orl > rlast) { rlast = orl; rv = orv; }
+          if (half == 0 && rlast >= 0)
+            atomicMax(&l_claim[cslot], ((unsigned long long)(unsigned)(rlast + 1) << 32) |
+                                           __float_as_uint(rv * kPlaneUnscale));
+        }
       }
     }
 #pragma unroll
@@ -773,12 +815,13 @@ __global__ __launch_bounds__(kPage32Threads) void gram_page_f32_kernel(GramArgs 
       float sv = half_sum(rsum[r]);
       int c = ccol[r];
       float v = cval[r];
-      last_claim_reduce(c, v);
+      if (wave_claims) last_claim_reduce(c, v);
       if (col == 0) {
         const int rslot = rb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-        l_sum[rslot] = sv;
+        l_sum[rslot] = sv * kPlaneUnscale;
         if (c >= 0)
-          atomicMax(&l_claim[rslot], ((unsigned long long)(unsigned)(c + 1) << 32) | __float_as_uint(v));
+          atomicMax(&l_claim[rslot], ((unsigned long long)(unsigned)(c + 1) << 32) |
+                                         __float_as_uint(v * kPlaneUnscale));
       }
     }
   }
