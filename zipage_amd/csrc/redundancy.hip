@@ -468,6 +468,8 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
   const int nd = n / 2 + (((n & 1) || ai < n / 2) ? 1 : 0);     // distances 0 .. nd-1
   const int tiles_per_page = p.BS / TN;
   const int ntiles = nd * tiles_per_page;
+  // tile / tiles_per_page without a division per tile (at most a few hundred tiles, a handful per page)
+  const int tpp_rcp = (65536 + tiles_per_page - 1) / tiles_per_page;
   const int dpieces = p.D / 4;
   const int64_t k_row = (int64_t)p.Hkv * p.D * 4;
   const char* kbase = p.k + (l * p.k_sl) * 4 + (int64_t)h * p.D * 4;
@@ -476,7 +478,7 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
   vec16 pre[STAGE_IT];
   auto col_page = [&](int d) { return ai + d < n ? ai + d : ai + d - n; };
   auto issue_loads = [&](int tile) {
-    const int d = tile / tiles_per_page, toff = (tile - d * tiles_per_page) * TN;
+    const int d = (tile * tpp_rcp) >> 16, toff = (tile - d * tiles_per_page) * TN;
     const char* src = kbase + (int64_t)vpage[col_page(d)] * p.k_sp * 4 + (int64_t)toff * k_row;
 #pragma unroll
     for (int i = 0; i < STAGE_IT; ++i) {
@@ -545,7 +547,7 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
   // the column sums of tile t are complete after the barrier that ends it: the waves' shares are
   // added in wave order and stored while tile t+1 is being multiplied
   auto finish_columns = [&](int tile) {
-    const int d = tile / tiles_per_page, toff = (tile - d * tiles_per_page) * TN;
+    const int d = (tile * tpp_rcp) >> 16, toff = (tile - d * tiles_per_page) * TN;
     if (d == 0 || tid >= TN) return;
     const float* pt = l_cpart + (tile & 1) * kSymWaves * TN;
     float v = pt[tid];
@@ -561,7 +563,7 @@ __global__ __launch_bounds__(kSymWaves * 64) void gram_raw_sym_f32_kernel(GramAr
     float* cur = (tile & 1) ? kbuf1 : kbuf0;
     float* nxt = (tile & 1) ? kbuf0 : kbuf1;
     if (tile + 1 < ntiles) issue_loads(tile + 1);
-    const int d = tile / tiles_per_page, toff = (tile - d * tiles_per_page) * TN;
+    const int d = (tile * tpp_rcp) >> 16, toff = (tile - d * tiles_per_page) * TN;
     const int jc = vidx[col_page(d)];
     float* cpart = l_cpart + ((tile & 1) * kSymWaves + wave) * TN;
 #pragma unroll
