@@ -9,12 +9,16 @@
 //     r_i = sum_j S_ij  -  sum_{j : c*(j) = i} S_ji .
 //
 // Kernels in this file:
-//   gram_kernel        fp32 caches, both variants: v_mfma_f32_32x32x2_f32 on keys divided by
-//                      their cache-dtype norm in fp32 (the reference's arithmetic), full
-//                      matrix, a wave owns 32 rows for all columns.
+//   gram_kernel        fp32 caches, both variants, any page size and table length:
+//                      v_mfma_f32_32x32x2_f32 on keys divided by their norm in fp32, full matrix,
+//                      a wave owns 32 rows for all columns.
 //   gram_page_f32_kernel  fp32 caches, lightning, pages of at most 256 keys: a workgroup walks the
-//                      pages of a row; the normalised page resident in LDS, one barrier, both
-//                      operands read from that copy, the next page requested under the tiles.
+//                      pages of a row; the normalised page resident in LDS as two fp16 planes per
+//                      element (fp32-grade products on the 16-bit matrix instructions), one
+//                      barrier, both operands read from that copy, every pair of key blocks once.
+//   gram_raw_sym_f32_kernel  fp32 caches, raw, pages of at most 256 keys and tables of at most 16
+//                      pages: every unordered pair of pages once, column tiles staged as the same
+//                      two planes.
 //   gram_split_kernel  16-bit caches, lightning with pages above 256 keys: normalised keys
 //                      split into two bf16 planes, three MFMAs per k-step, full matrix.
 //   gram_page_kernel   16-bit caches, lightning: a workgroup walks the pages of one (layer,
