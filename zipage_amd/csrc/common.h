@@ -30,12 +30,24 @@ void zp_set_error(const char* fmt, ...);
     }                                                                  \
   } while (0)
 
-// Scratch zp_attention_score cannot do without (it takes the three-sweep kernel when the caller
-// brings less than zp_attention_score_workspace() asks for).  Library-internal.
+// The scratch the one-sweep scorer of one cache dtype asks for (declared in the header too).
 extern "C" int64_t zp_attention_score_workspace_for(int32_t L, int32_t B, int32_t NB, int32_t BS,
                                                     int32_t Hkv, int32_t Hq, int32_t W, int32_t dtype);
+// Scratch zp_attention_score cannot do without (it takes the three-sweep kernel when the caller
+// brings less than zp_attention_score_workspace() asks for).  Library-internal.
 int64_t zp_attention_score_workspace_floor(int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
                                            int32_t Hq, int32_t W);
+// gather.hip, library-internal: K/V compaction and the carried scores' compaction in one launch
+// where the shapes allow it (zp_compress_kv followed by zp_compress_score otherwise); the
+// arguments of the two.
+int zp_compress_kv_and_score(void* key, void* value, void* score_cache, const void* scores_src,
+                             const uint8_t* flag, const int32_t* block_table,
+                             const int32_t* target_block_table, int32_t L, int32_t B, int32_t NB,
+                             int32_t BS, int32_t Hkv, int32_t D, int32_t num_pages,
+                             int32_t target_width, int64_t k_sl, int64_t k_sp, int64_t k_ss,
+                             int64_t k_sh, int64_t v_sl, int64_t v_sp, int64_t v_ss, int64_t v_sh,
+                             int64_t c_sl, int64_t c_sp, int64_t c_ss, int64_t c_sh, int32_t dtype,
+                             void* stream);
 
 // ---------------------------------------------------------------- element types
 // Storage element tags.  bf16/fp16 are kept as raw 16-bit patterns in memory.

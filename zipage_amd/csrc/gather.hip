@@ -13,7 +13,10 @@
 // barrier orders load-before-store) or in an earlier round.  Later rounds only read
 // positions > every position written so far, so rounds need no ordering between them
 // and the next round's loads overlap the current round's stores.
+// The one-call pipeline moves the carried scores of the survivors in the same launch (same list,
+// rounds of their own after the K/V rounds); zp_compress_score is the launch of its own.
 #include "common.h"
+#include <type_traits>
 
 namespace {
 
@@ -60,6 +63,11 @@ struct CompactArgs {
   // score compaction only: when set, the value of logical token s of row (l, b, h) is read from
   // rows[((l*B + b)*Hkv + h)*T + s] (elements of sizeof(P)) instead of from `a` through the table
   const char* rows;
+  // K/V compaction with the carried scores in the same launch (CES != 0): the score cache, its
+  // byte strides, and optionally the rows to read the scores from (as `rows` above)
+  char* c;
+  const char* c_rows;
+  int64_t c_sl, c_sp, c_ss, c_sh;
 };
 
 // Survivors are written once and not read again by this kernel: non-temporal stores keep them
@@ -68,7 +76,8 @@ struct CompactArgs {
 #define ZP_NT_LOAD(ptr) (*(ptr))
 #define ZP_NT_STORE(v, ptr) __builtin_nontemporal_store(v, ptr)
 // POW2: page size and pieces-per-vector are powers of two, so every index split is a shift.
-template <typename P, int R, bool HAS_B, bool POW2>
+// CES: bytes of a carried-score element moved along with K and V by the same survivor list (0: none).
+template <typename P, int R, bool HAS_B, bool POW2, int CES = 0>
 __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
   extern __shared__ __align__(16) char smem[];
   __shared__ int scan_lds[kThreads / 64];
@@ -153,6 +162,37 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
       }
     }
   }
+  if constexpr (CES != 0) {
+    // the carried score of every survivor follows its key: same list, same gather -> barrier ->
+    // scatter rounds (the score cache aliases its own targets exactly as the key cache does)
+    typedef typename std::conditional<CES == 4, uint32_t, uint16_t>::type E;
+    constexpr int RC = 4;
+    char* cbase = p.c + l * p.c_sl + h * p.c_sh;
+    for (int base = 0; base < total; base += kThreads * RC) {
+      E rc[RC];
+#pragma unroll
+      for (int r = 0; r < RC; ++r) {
+        const int s = list[min(base + r * kThreads + tid, total - 1)];
+        if (p.c_rows) {
+          rc[r] = *(const E*)(p.c_rows + ((int64_t)item * T + s) * CES);
+        } else {
+          const int j = page_of(s), slot = s - j * p.BS;
+          rc[r] = *(const E*)(cbase + (int64_t)tab[j] * p.c_sp + slot * p.c_ss);
+        }
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+#pragma unroll
+      for (int r = 0; r < RC; ++r) {
+        const int i = base + r * kThreads + tid;
+        if (i < total) {
+          const int j = page_of(i), slot = i - j * p.BS;
+          const int64_t pid = tgt[j];
+          if (pid >= 0) *(E*)(cbase + pid * p.c_sp + slot * p.c_ss) = rc[r];
+        }
+      }
+    }
+  }
 }
 
 static int log2_exact(int v) {
@@ -162,31 +202,31 @@ static int log2_exact(int v) {
   return s;
 }
 
-template <typename P, int R, bool HAS_B, bool POW2>
+template <typename P, int R, bool HAS_B, bool POW2, int CES = 0>
 int launch_compact_impl(CompactArgs a, int L, hipStream_t st) {
   a.n_items = L * a.B * a.Hkv;
   const int T = a.NB * a.BS;
   size_t smem = (((size_t)T * 2 + 15) & ~(size_t)15) + sizeof(int) * (a.NB + a.target_width);
   dim3 grid((unsigned)((int64_t)L * a.B * a.Hkv));
   if (smem > 64 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)compact_kernel<P, R, HAS_B, POW2>,
+    hipError_t e = hipFuncSetAttribute((const void*)compact_kernel<P, R, HAS_B, POW2, CES>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
     if (e != hipSuccess) {
       zp_set_error("compaction: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
       return ZP_EHIP;
     }
   }
-  hipLaunchKernelGGL((compact_kernel<P, R, HAS_B, POW2>), grid, dim3(kThreads), smem, st, a);
+  hipLaunchKernelGGL((compact_kernel<P, R, HAS_B, POW2, CES>), grid, dim3(kThreads), smem, st, a);
   ZP_LAUNCH_CHECK();
   return ZP_OK;
 }
 
-template <typename P, int R, bool HAS_B>
+template <typename P, int R, bool HAS_B, int CES = 0>
 int launch_compact(CompactArgs a, int L, hipStream_t st) {
   a.lpv_shift = log2_exact(a.lpv);
   a.bs_shift = log2_exact(a.BS);
-  if (a.lpv_shift >= 0 && a.bs_shift >= 0) return launch_compact_impl<P, R, HAS_B, true>(a, L, st);
-  return launch_compact_impl<P, R, HAS_B, false>(a, L, st);
+  if (a.lpv_shift >= 0 && a.bs_shift >= 0) return launch_compact_impl<P, R, HAS_B, true, CES>(a, L, st);
+  return launch_compact_impl<P, R, HAS_B, false, CES>(a, L, st);
 }
 
 inline bool aligned_to(int64_t v, int n) { return (v % n) == 0; }
@@ -210,13 +250,17 @@ __global__ __launch_bounds__(kThreads) void store_query_kernel(
 
 }  // namespace
 
-extern "C" int zp_compress_kv(void* key, void* value, const uint8_t* flag,
-                              const int32_t* block_table, const int32_t* target_block_table,
-                              int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
-                              int32_t D, int32_t num_pages, int32_t target_width,
-                              int64_t k_sl, int64_t k_sp, int64_t k_ss, int64_t k_sh,
-                              int64_t v_sl, int64_t v_sp, int64_t v_ss, int64_t v_sh,
-                              int32_t dtype, void* stream) {
+namespace {
+// K/V compaction; with score_cache != nullptr the carried scores move in the same launch when the
+// K/V vectors allow 16-byte pieces (otherwise *fused is left false and the caller runs
+// zp_compress_score itself).
+int compress_kv_impl(void* key, void* value, const uint8_t* flag, const int32_t* block_table,
+                     const int32_t* target_block_table, int32_t L, int32_t B, int32_t NB, int32_t BS,
+                     int32_t Hkv, int32_t D, int32_t num_pages, int32_t target_width, int64_t k_sl,
+                     int64_t k_sp, int64_t k_ss, int64_t k_sh, int64_t v_sl, int64_t v_sp,
+                     int64_t v_ss, int64_t v_sh, int32_t dtype, void* score_cache,
+                     const void* scores_src, int64_t c_sl, int64_t c_sp, int64_t c_ss, int64_t c_sh,
+                     bool* fused, void* stream) {
   ZP_REQUIRE(key && value && flag && block_table && target_block_table, "compress_kv: null pointer");
   ZP_REQUIRE(L >= 0 && B >= 0 && NB > 0 && BS > 0 && Hkv > 0 && D > 0 && target_width > 0,
              "compress_kv: bad dims L=%d B=%d NB=%d BS=%d Hkv=%d D=%d tw=%d", L, B, NB, BS, Hkv, D,
@@ -225,6 +269,7 @@ extern "C" int zp_compress_kv(void* key, void* value, const uint8_t* flag,
   ZP_REQUIRE((int64_t)NB * BS <= 65536, "compress_kv: NB*BS=%lld exceeds 65536",
              (long long)NB * BS);
   ZP_REQUIRE((int64_t)L * B * Hkv < ((int64_t)1 << 31), "compress_kv: too many (layer, sequence, head) rows");
+  if (fused) *fused = false;
   if (L == 0 || B == 0) return ZP_OK;
   const int es = zp_dtype_bytes(dtype);
   CompactArgs a;
@@ -234,6 +279,8 @@ extern "C" int zp_compress_kv(void* key, void* value, const uint8_t* flag,
   a.target_width = target_width;
   a.a_sl = k_sl * es; a.a_sp = k_sp * es; a.a_ss = k_ss * es; a.a_sh = k_sh * es;
   a.b_sl = v_sl * es; a.b_sp = v_sp * es; a.b_ss = v_ss * es; a.b_sh = v_sh * es;
+  a.c = (char*)score_cache; a.c_rows = (const char*)scores_src;
+  a.c_sl = c_sl * es; a.c_sp = c_sp * es; a.c_ss = c_ss * es; a.c_sh = c_sh * es;
   const int64_t vec = (int64_t)D * es;
   int piece = 2;
   for (int cand : {16, 8, 4}) {
@@ -247,11 +294,50 @@ extern "C" int zp_compress_kv(void* key, void* value, const uint8_t* flag,
   ZP_REQUIRE((int64_t)target_width * BS * a.lpv < (int64_t)1 << 31, "compress_kv: row too large");
   hipStream_t st = (hipStream_t)stream;
   switch (piece) {
-    case 16: return launch_compact<u32x4, kCompactR, true>(a, L, st);
+    case 16:
+      if (score_cache && fused) {
+        *fused = true;
+        if (es == 4) return launch_compact<u32x4, kCompactR, true, 4>(a, L, st);
+        return launch_compact<u32x4, kCompactR, true, 2>(a, L, st);
+      }
+      return launch_compact<u32x4, kCompactR, true>(a, L, st);
     case 8:  return launch_compact<u32x2, 8, true>(a, L, st);
     case 4:  return launch_compact<uint32_t, 8, true>(a, L, st);
     default: return launch_compact<uint16_t, 8, true>(a, L, st);
   }
+}
+}  // namespace
+
+extern "C" int zp_compress_kv(void* key, void* value, const uint8_t* flag,
+                              const int32_t* block_table, const int32_t* target_block_table,
+                              int32_t L, int32_t B, int32_t NB, int32_t BS, int32_t Hkv,
+                              int32_t D, int32_t num_pages, int32_t target_width,
+                              int64_t k_sl, int64_t k_sp, int64_t k_ss, int64_t k_sh,
+                              int64_t v_sl, int64_t v_sp, int64_t v_ss, int64_t v_sh,
+                              int32_t dtype, void* stream) {
+  return compress_kv_impl(key, value, flag, block_table, target_block_table, L, B, NB, BS, Hkv, D,
+                          num_pages, target_width, k_sl, k_sp, k_ss, k_sh, v_sl, v_sp, v_ss, v_sh,
+                          dtype, nullptr, nullptr, 0, 0, 0, 0, nullptr, stream);
+}
+
+// K/V compaction and the compaction of the carried scores (zp_compress_score with the same flags
+// and tables) as one launch where the shapes allow it, as the two calls otherwise.
+int zp_compress_kv_and_score(void* key, void* value, void* score_cache, const void* scores_src,
+                             const uint8_t* flag, const int32_t* block_table,
+                             const int32_t* target_block_table, int32_t L, int32_t B, int32_t NB,
+                             int32_t BS, int32_t Hkv, int32_t D, int32_t num_pages,
+                             int32_t target_width, int64_t k_sl, int64_t k_sp, int64_t k_ss,
+                             int64_t k_sh, int64_t v_sl, int64_t v_sp, int64_t v_ss, int64_t v_sh,
+                             int64_t c_sl, int64_t c_sp, int64_t c_ss, int64_t c_sh, int32_t dtype,
+                             void* stream) {
+  ZP_REQUIRE(score_cache, "compress_kv_and_score: null score cache");
+  bool fused = false;
+  int rc = compress_kv_impl(key, value, flag, block_table, target_block_table, L, B, NB, BS, Hkv, D,
+                            num_pages, target_width, k_sl, k_sp, k_ss, k_sh, v_sl, v_sp, v_ss, v_sh,
+                            dtype, score_cache, scores_src, c_sl, c_sp, c_ss, c_sh, &fused, stream);
+  if (rc != ZP_OK || fused) return rc;
+  return zp_compress_score(score_cache, scores_src, flag, block_table, target_block_table, L, B, NB,
+                           BS, Hkv, num_pages, target_width, c_sl, c_sp, c_ss, c_sh, dtype, stream);
 }
 
 extern "C" int zp_compress_score(void* score_cache, const void* scores_src, const uint8_t* flag,
@@ -277,6 +363,7 @@ extern "C" int zp_compress_score(void* score_cache, const void* scores_src, cons
   a.target_width = target_width; a.lpv = 1;
   a.a_sl = c_sl * es; a.a_sp = c_sp * es; a.a_ss = c_ss * es; a.a_sh = c_sh * es;
   a.b_sl = a.b_sp = a.b_ss = a.b_sh = 0;
+  a.c = nullptr; a.c_rows = nullptr; a.c_sl = a.c_sp = a.c_ss = a.c_sh = 0;
   hipStream_t st = (hipStream_t)stream;
   if (es == 4) return launch_compact<uint32_t, 4, false>(a, L, st);
   return launch_compact<uint16_t, 4, false>(a, L, st);

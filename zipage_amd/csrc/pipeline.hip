@@ -230,18 +230,21 @@ int run_layers(void* k_cache, void* v_cache, const void* query_cache, void* scor
     t.stop(ZP_STAGE_TOPK_MASK);
   }
 
+  // with a carried score cache the scores of the survivors move in the K/V launch (the stage events
+  // of the score compaction are then recorded back to back: its time is inside compress_kv)
   t.start(ZP_STAGE_COMPRESS_KV);
-  rc = zp_compress_kv(k_cache, v_cache, flag, block_table, target, L, B, NB, BS, Hkv, D,
-                      num_pages, target_width, k_sl, k_sp, k_ss, k_sh, v_sl, v_sp, v_ss, v_sh,
-                      dtype, stream);
+  if (glob)
+    rc = zp_compress_kv_and_score(k_cache, v_cache, score_cache, carried, flag, block_table, target, L,
+                                  B, NB, BS, Hkv, D, num_pages, target_width, k_sl, k_sp, k_ss, k_sh,
+                                  v_sl, v_sp, v_ss, v_sh, c_sl, c_sp, c_ss, c_sh, dtype, stream);
+  else
+    rc = zp_compress_kv(k_cache, v_cache, flag, block_table, target, L, B, NB, BS, Hkv, D,
+                        num_pages, target_width, k_sl, k_sp, k_ss, k_sh, v_sl, v_sp, v_ss, v_sh,
+                        dtype, stream);
   if (rc != ZP_OK) return rc;
   t.stop(ZP_STAGE_COMPRESS_KV);
-
   if (glob) {
     t.start(ZP_STAGE_COMPRESS_SCORE);
-    rc = zp_compress_score(score_cache, carried, flag, block_table, target, L, B, NB, BS, Hkv,
-                           num_pages, target_width, c_sl, c_sp, c_ss, c_sh, dtype, stream);
-    if (rc != ZP_OK) return rc;
     t.stop(ZP_STAGE_COMPRESS_SCORE);
   }
   return ZP_OK;
