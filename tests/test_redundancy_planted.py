@@ -92,6 +92,8 @@ def planted_case(seed, dtype, nb_choices=(3, 4), B=2, L=1):
                     else:
                         plant(a, d, c)
                 plan[(l, b, h)] = triples
+    if dtype == torch.float32:     # fp32 norms are not rounded to a coarser type
+        return k, enc, tables, plan
     return _clear_of_norm_boundaries(k.to(dtype)), enc, tables, plan
 
 
@@ -221,6 +223,35 @@ def test_planted_pairs_against_oracle(dev, dtype, variant, thr):
     _close_in_ulps(gl, wl, dtype, ulps=1, frac_exact=0.97,
                    chain_scale=chain_scale if variant == "raw" else None)
     _close_in_ulps(gr, wr, dtype, ulps=4, frac_exact=0.5)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("variant", ["lightning", "raw"])
+@pytest.mark.parametrize("thr", [THR, -0.1])
+def test_planted_pairs_fp32(dev, variant, thr):
+    """fp32 caches on the same data: most 32 x 32 tiles hold no entry over the threshold and take
+    the kernels' short path, the planted ones take the claim path; a claim moves its row by its
+    cosine (>= 0.51), the comparison allows 1e-3."""
+    from zipage_amd import kernel as K
+    k, enc, tables, plan = planted_case(107, torch.float32)
+    kw = dict(threshold=thr, temperature=0.4, return_logits=True)
+    if variant == "lightning":
+        wl, wr = O.lightning_redudancy_score(k, enc, **kw)
+        noclaim = O.lightning_redudancy_logits(k, enc, 2.0)
+        gl, gr = K.lightning_redudancy_score(k.to(dev), enc.to(dev), **kw)
+    else:
+        wl, wr = O.raw_redudancy_score(k, enc, **kw)
+        noclaim = O.raw_redudancy_logits(k, enc, 2.0)
+        gl, gr = K.raw_redudancy_score(k.to(dev), enc.to(dev), **kw)
+    fin = torch.isfinite(wl)
+    if thr > 0:
+        moved = ((noclaim.reshape(-1) - wl.reshape(-1)).abs() > 0.4) & fin.reshape(-1)
+        assert int(moved.sum()) >= 2 * 12 * HKV, f"only {int(moved.sum())} rows carry a claim"
+    gl, gr = gl.cpu(), gr.cpu()
+    assert torch.equal(torch.isfinite(gl), fin)
+    err = (gl[fin] - wl[fin]).abs().max().item()
+    assert err < 1e-3, f"row sums off by {err}"
+    assert torch.allclose(gr, wr, rtol=1e-3, atol=1e-9)
 
 
 # rounding chain of the all-pairs variant the GPU kernel is held to: the reference's partial sums
