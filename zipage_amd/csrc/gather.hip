@@ -22,6 +22,7 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kCompactR = 8;   // 16-byte pieces each thread gathers per round
+constexpr int kSplitKvRows = 1024;   // up to this many (layer, sequence, head) rows K and V get workgroups of their own
 // native vector types keep the staged pieces in VGPRs
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -68,6 +69,9 @@ struct CompactArgs {
   char* c;
   const char* c_rows;
   int64_t c_sl, c_sp, c_ss, c_sh;
+  // !HAS_B with split_kv: the grid is twice n_items; workgroups n_items .. 2 n_items - 1 move
+  // `b` (the values) with the same list, the first n_items move `a` (and the carried scores)
+  int split_kv;
 };
 
 // Survivors are written once and not read again by this kernel: non-temporal stores keep them
@@ -91,7 +95,8 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
   // works on one head's 256-byte slice of the token rows.  Measured against giving each XCD a
   // contiguous range of items (all heads of a sequence on one XCD: 2.5 % slower) and against
   // rotating the head index by the sequence index (4 % slower), inside one allocation.
-  const int item = blockIdx.x;
+  const int which = (!HAS_B && p.split_kv && (int)blockIdx.x >= p.n_items) ? 1 : 0;
+  const int item = (int)blockIdx.x - which * p.n_items;
   if (item >= p.n_items) return;
   const int h = item % p.Hkv;
   const int b = (item / p.Hkv) % p.B;
@@ -125,8 +130,9 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
 
   // ---- phase 2: gather -> barrier -> scatter, R pieces per thread per round
   const int units = total * p.lpv;
-  char* abase = p.a + l * p.a_sl + h * p.a_sh;
+  char* abase = which ? p.b + l * p.b_sl + h * p.b_sh : p.a + l * p.a_sl + h * p.a_sh;
   char* bbase = HAS_B ? p.b + l * p.b_sl + h * p.b_sh : nullptr;
+  const int64_t a_sp = which ? p.b_sp : p.a_sp, a_ss = which ? p.b_ss : p.a_ss;
   for (int base = 0; base < units; base += kThreads * R) {
     P ra[R];
     P rb[R];
@@ -141,7 +147,7 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
       if (!HAS_B && p.rows)
         ra[r] = *(const P*)(p.rows + ((int64_t)item * T + s) * (int)sizeof(P));
       else
-        ra[r] = ZP_NT_LOAD((const P*)(abase + pid * p.a_sp + slot * p.a_ss + piece * (int)sizeof(P)));
+        ra[r] = ZP_NT_LOAD((const P*)(abase + pid * a_sp + slot * a_ss + piece * (int)sizeof(P)));
       if (HAS_B)
         rb[r] = ZP_NT_LOAD((const P*)(bbase + pid * p.b_sp + slot * p.b_ss + piece * (int)sizeof(P)));
     }
@@ -155,14 +161,14 @@ __global__ __launch_bounds__(kThreads) void compact_kernel(CompactArgs p) {
         const int j = page_of(i), slot = i - j * p.BS;
         const int64_t pid = tgt[j];
         if (pid >= 0) {
-          ZP_NT_STORE(ra[r], (P*)(abase + pid * p.a_sp + slot * p.a_ss + piece * (int)sizeof(P)));
+          ZP_NT_STORE(ra[r], (P*)(abase + pid * a_sp + slot * a_ss + piece * (int)sizeof(P)));
           if (HAS_B)
             ZP_NT_STORE(rb[r], (P*)(bbase + pid * p.b_sp + slot * p.b_ss + piece * (int)sizeof(P)));
         }
       }
     }
   }
-  if constexpr (CES != 0) {
+  if (CES != 0 && which == 0) {
     // the carried score of every survivor follows its key: same list, same gather -> barrier ->
     // scatter rounds (the score cache aliases its own targets exactly as the key cache does)
     typedef typename std::conditional<CES == 4, uint32_t, uint16_t>::type E;
@@ -207,7 +213,7 @@ int launch_compact_impl(CompactArgs a, int L, hipStream_t st) {
   a.n_items = L * a.B * a.Hkv;
   const int T = a.NB * a.BS;
   size_t smem = (((size_t)T * 2 + 15) & ~(size_t)15) + sizeof(int) * (a.NB + a.target_width);
-  dim3 grid((unsigned)((int64_t)L * a.B * a.Hkv));
+  dim3 grid((unsigned)((int64_t)L * a.B * a.Hkv * (!HAS_B && a.split_kv ? 2 : 1)));
   if (smem > 64 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)compact_kernel<P, R, HAS_B, POW2, CES>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -293,12 +299,26 @@ int compress_kv_impl(void* key, void* value, const uint8_t* flag, const int32_t*
   a.lpv = (int)(vec / piece);
   ZP_REQUIRE((int64_t)target_width * BS * a.lpv < (int64_t)1 << 31, "compress_kv: row too large");
   hipStream_t st = (hipStream_t)stream;
+  a.split_kv = 0;
+  // few rows: keys and values go to workgroups of their own (twice the workgroups per CU to hide
+  // the gather's latency: 0.340 against 0.347 ms per step at 64 sequences x 8 heads; with many rows
+  // the CUs are full either way and one survivor list per row is cheaper)
+  const bool split = piece == 16 && (int64_t)L * B * Hkv <= kSplitKvRows;
   switch (piece) {
     case 16:
       if (score_cache && fused) {
         *fused = true;
+        if (split) {
+          a.split_kv = 1;
+          if (es == 4) return launch_compact<u32x4, 2 * kCompactR, false, 4>(a, L, st);
+          return launch_compact<u32x4, 2 * kCompactR, false, 2>(a, L, st);
+        }
         if (es == 4) return launch_compact<u32x4, kCompactR, true, 4>(a, L, st);
         return launch_compact<u32x4, kCompactR, true, 2>(a, L, st);
+      }
+      if (split) {
+        a.split_kv = 1;
+        return launch_compact<u32x4, 2 * kCompactR, false>(a, L, st);
       }
       return launch_compact<u32x4, kCompactR, true>(a, L, st);
     case 8:  return launch_compact<u32x2, 8, true>(a, L, st);
@@ -364,6 +384,7 @@ extern "C" int zp_compress_score(void* score_cache, const void* scores_src, cons
   a.a_sl = c_sl * es; a.a_sp = c_sp * es; a.a_ss = c_ss * es; a.a_sh = c_sh * es;
   a.b_sl = a.b_sp = a.b_ss = a.b_sh = 0;
   a.c = nullptr; a.c_rows = nullptr; a.c_sl = a.c_sp = a.c_ss = a.c_sh = 0;
+  a.split_kv = 0;
   hipStream_t st = (hipStream_t)stream;
   if (es == 4) return launch_compact<uint32_t, 4, false>(a, L, st);
   return launch_compact<uint16_t, 4, false>(a, L, st);
