@@ -22,7 +22,10 @@ namespace {
 
 constexpr int kThreads = 256;
 constexpr int kCompactR = 8;   // 16-byte pieces each thread gathers per round
-constexpr int kSplitKvRows = 1024;   // up to this many (layer, sequence, head) rows K and V get workgroups of their own
+#ifndef ZP_SPLIT_ROWS
+#define ZP_SPLIT_ROWS 1024
+#endif
+constexpr int kSplitKvRows = ZP_SPLIT_ROWS;   // up to this many (layer, sequence, head) rows K and V get workgroups of their own
 // native vector types keep the staged pieces in VGPRs
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
