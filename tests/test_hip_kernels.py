@@ -100,6 +100,37 @@ def test_compress_kv_bit_exact(dev, dtype, style):
     assert torch.equal(gv.cpu().view(torch.uint8), wv.view(torch.uint8))
 
 
+@pytest.mark.parametrize("style", ["aliased", "cow"])
+def test_compress_kv_many_rows(dev, style):
+    """More than 1 024 (layer, sequence, head) rows: one workgroup per row moves keys and values
+    (with fewer rows, as in every other small test, keys and values get workgroups of their own)."""
+    from zipage_amd.kernel import compress_kv
+    dtype = torch.bfloat16
+    L, B, Hkv, BS, D, P = 3, 44, 8, 64, 32, 300
+    assert L * B * Hkv > 1024
+    s = _setup(17, dtype, L=L, B=B, Hkv=Hkv, Hq=Hkv, D=D, BS=BS, W=16, nb_choices=(3, 4, 5), budget=2,
+               num_pages=P)
+    k, v, enc = s["k"], s["v"], s["enc"]
+    NB = enc.shape[1]
+    g = torch.Generator().manual_seed(19)
+    scores = O.pad_mask(torch.rand((L, B, Hkv, NB, BS), generator=g), enc).view(L, B, Hkv, NB * BS)
+    flag = O.topk_mask(scores, 2 * BS).view(L, B, Hkv, NB, BS)
+    if style == "aliased":
+        target = s["target"]
+    else:
+        used = cases.touched_pages(enc)
+        fresh = [p for p in range(P) if p not in used]
+        assert len(fresh) >= 2 * B
+        target = torch.tensor([[fresh[2 * b], fresh[2 * b + 1], t[2]] for b, t in enumerate(s["tables"])],
+                              dtype=torch.int32)
+    wk, wv = k.clone(), v.clone()
+    O.compress_kv_loop(wk, wv, flag, enc, target)
+    gk, gv = k.clone().to(dev), v.clone().to(dev)
+    compress_kv(gk, gv, flag.to(dev), enc.to(dev), target.to(dev))
+    assert torch.equal(gk.cpu().view(torch.uint8), wk.view(torch.uint8))
+    assert torch.equal(gv.cpu().view(torch.uint8), wv.view(torch.uint8))
+
+
 def test_compress_kv_strided_views(dev):
     """key/value as slices of one (2, L, pages, BS, Hkv, D) allocation, layer-sliced."""
     from zipage_amd.kernel import compress_kv

@@ -64,6 +64,37 @@ def test_one_call_equals_separate_stages(dev, dtype, name, deterministic_carry):
     assert (outs[0][0].flatten(3).sum(-1) == 2 * 256).all()
 
 
+@pytest.mark.parametrize("deterministic_carry", [True, False])
+def test_one_call_equals_separate_stages_on_many_rows(dev, deterministic_carry):
+    """More than 1 024 (layer, sequence, head) rows with a carried score cache: the compaction
+    launch is then the one-workgroup-per-row kernel with the scores' rounds behind the K/V rounds
+    (every other test here stays below and gets keys and values in workgroups of their own)."""
+    from zipage_amd.compress import CompressConfig, StageTimer, compress_layers
+    dtype, L, B, Hkv, Hq, D, BS, W, P = torch.bfloat16, 2, 66, 8, 8, 64, 128, 16, 420
+    assert L * B * Hkv > 1024
+    tables, enc, target = cases.random_tables(93, B, P, [3, 4], 2)
+    k, v, q, sc = cases.make_caches(93, L, P, BS, Hkv, Hq, D, W, B + 1, dtype,
+                                    touched=cases.touched_pages(enc), with_score_cache=True)
+    base = torch.randn((1, 1, 1, Hkv, D), generator=torch.Generator().manual_seed(94))
+    k = (k.float() * 0.8 + 0.6 * base).to(dtype)
+    qid = torch.arange(B, dtype=torch.int32)
+    comp = torch.tensor([b % 2 == 1 for b in range(B)])
+    cfg = CompressConfig(budget_blocks=2, query_cache_len=W, **SWITCHES["scripts"])
+    outs = []
+    for one_call in (True, False):
+        gk, gv, gsc = k.clone().to(dev), v.clone().to(dev), sc.clone().to(dev)
+        res = compress_layers(gk, gv, q.to(dev), gsc, qid.to(dev), enc.to(dev), comp.to(dev),
+                              target.to(dev), cfg, timer=StageTimer(False),
+                              return_intermediates=not one_call,
+                              deterministic_carry=deterministic_carry)
+        torch.cuda.synchronize()
+        flag = res if one_call else res[0]
+        outs.append((flag.cpu(), gk.cpu(), gv.cpu(), gsc.cpu()))
+    for a, b in zip(*outs):
+        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8))
+    assert (outs[0][0].flatten(3).sum(-1) == 2 * BS).all()
+
+
 def test_one_call_rejects_a_short_workspace(dev):
     import ctypes
     from zipage_amd import _lib
