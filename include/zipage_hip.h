@@ -210,8 +210,9 @@ int zp_compress_score(void* score_cache, const void* scores_src, const uint8_t* 
  * The body of ModelRunner.compress for one chunk of layers
  * (zipage/engine/model_runner.py:466-622): attention_score -> [max-norm, global_score] ->
  * [redundancy] -> pooling / combine / sink / window mask / pad mask / top-k -> compress_kv ->
- * [compress_score], enqueued on `stream` in that order by the entry points above, so every
- * result is bit-identical to calling them one after the other.  The switches are the fields of
+ * [compress_score], enqueued on `stream` in that order, so every result is bit-identical to
+ * calling the entry points above one after the other (the carried scores of the survivors move
+ * inside the compress_kv launch, by the same survivor list).  The switches are the fields of
  * zipage/config.py:22-46 that the runner reads. */
 typedef struct {
   int32_t budget_blocks;          /* max_cache_blocks_per_seq: k = BS * budget_blocks survive */
