@@ -365,8 +365,11 @@ def main():
     ap.add_argument("--no-extra-legs", action="store_true",
                     help="skip the 64-sequence leg and the end-to-end leg that follow the default run")
     ap.add_argument("--no-e2e-variants", action="store_true",
-                    help="skip the four shorter end-to-end runs (reference scripts' switches / ragged "
-                         "prompts, each with side-stream and in-line compression)")
+                    help="skip the shorter end-to-end runs that follow the end-to-end leg (ragged "
+                         "prompts with side-stream and with in-line compression)")
+    ap.add_argument("--all-e2e-variants", action="store_true",
+                    help="also run the pair with the reference scripts' switch set (side stream and "
+                         "in line; ~90 s more)")
     ap.add_argument("--variant-tokens", type=int, default=2560,
                     help="greedy tokens per request in the end-to-end variants")
     ap.add_argument("--requests", type=int, default=256)
@@ -457,13 +460,15 @@ def main():
                                            not args.sync_compress, args.ragged_prompts,
                                            args.script_switches)
             if not args.no_e2e_variants:
-                # where overlap can exist and where the compression does more work: the reference
-                # scripts' switch set and ragged prompts, each on the side stream and in line,
-                # from this same process (shorter runs: every sequence still compresses 2-4 times)
+                # where overlap can exist: ragged prompts, on the side stream and in line, from this
+                # same process (shorter runs: every sequence still compresses 2-4 times); with
+                # --all-e2e-variants also where the compression does more work (the reference
+                # scripts' switch set)
                 n = min(args.out_tokens, args.variant_tokens)
+                pairs = ((True, False), (False, True)) if args.all_e2e_variants else ((False, True),)
                 out["end_to_end"]["variants"] = [
                     end_to_end(args.requests, args.prompt, n, a, ragged, scripts, attention_probe=False)
-                    for scripts, ragged in ((True, False), (False, True)) for a in (True, False)]
+                    for scripts, ragged in pairs for a in (True, False)]
     print(json.dumps(out))
 
 
